@@ -1,5 +1,5 @@
-"""Model families: Llama-3 (8B / 70B), Mixtral-8x7B (TP/EP-aware), Sapapel and Kivezen (single GPU)."""
-from .config import PRESETS, KivezenConfig, ModelConfig, SapapelConfig, get_config
+"""Model families: Llama-3 (8B / 70B), Mixtral-8x7B (TP/EP-aware), Sapapel, Kivezen and Nopunex (single GPU)."""
+from .config import PRESETS, KivezenConfig, ModelConfig, NopunexConfig, SapapelConfig, get_config
 from .llama import LlamaForCausalLM
 
 
@@ -10,10 +10,13 @@ def build_model(cfg, st, dtype, device):
     if isinstance(cfg, KivezenConfig):
         from .kivezen import KivezenForCausalLM
         return KivezenForCausalLM(cfg, st, dtype, device)
+    if isinstance(cfg, NopunexConfig):
+        from .nopunex import NopunexForCausalLM
+        return NopunexForCausalLM(cfg, st, dtype, device)
     if cfg.is_moe:
         from .mixtral import MixtralForCausalLM
         return MixtralForCausalLM(cfg, st, dtype, device)
     return LlamaForCausalLM(cfg, st, dtype, device)
 
 
-__all__ = ["PRESETS", "ModelConfig", "SapapelConfig", "KivezenConfig", "get_config", "LlamaForCausalLM", "build_model"]
+__all__ = ["PRESETS", "ModelConfig", "SapapelConfig", "KivezenConfig", "NopunexConfig", "get_config", "LlamaForCausalLM", "build_model"]

@@ -88,12 +88,21 @@ PRESETS: Dict[str, ModelConfig] = {
 
 @dataclasses.dataclass(frozen=True)
 class LatentAttentionSpec:
-    """Attention whose keys and values are expanded from one cached low-rank latent per token."""
+    """Attention whose keys and values are expanded from one cached low-rank latent per token.
+    Optional parts (0 / None: absent): queries through a normed latent of ``q_rank`` numbers; one
+    rotated key part of ``rot_dim`` numbers per token shared by all heads (cached beside the
+    latent) against ``rot_dim`` rotated query numbers per head; a sliding window of ``window``
+    positions; one learned sink logit per head in the softmax denominator."""
     heads: int
-    dim: int        # query / key size per head
+    dim: int        # unrotated query / key size per head
     vdim: int       # value size per head
     kv_rank: int    # size of the cached latent
     scale: float
+    q_rank: int = 0
+    rot_dim: int = 0
+    rot: Optional["RotarySpec"] = None
+    window: int = 0
+    sink: bool = False
 
 
 @dataclasses.dataclass(frozen=True)
@@ -177,12 +186,14 @@ class SapapelConfig:
 
 @dataclasses.dataclass(frozen=True)
 class RotarySpec:
-    """Rotation of interleaved coordinate pairs (2i, 2i+1) of the first ``dims`` coordinates by
-    position * base^(-2i/dims); ``scaling`` = (factor, original, fast, slow) stretches the slow
-    pairs (YaRN) and scales cos / sin by 0.1 ln(factor) + 1."""
+    """Rotation of coordinate pairs of the first ``dims`` coordinates by position * base^(-2i/dims):
+    pair i is (2i, 2i+1) (``halves`` False) or (i, i + dims/2) (``halves`` True); ``scaling`` =
+    (factor, original, fast, slow) stretches the slow pairs (YaRN) and scales cos / sin by
+    0.1 ln(factor) + 1."""
     dims: int
     base: float
     scaling: Optional[tuple] = None
+    halves: bool = False
 
 
 @dataclasses.dataclass(frozen=True)
@@ -343,8 +354,187 @@ class KivezenConfig:
                    streams=streams, loop=loop, logit_softcap=50.0)
 
 
+@dataclasses.dataclass(frozen=True)
+class DiffAttentionSpec:
+    """Grouped-query differential attention: two softmax maps per head over the same values, the
+    second subtracted with one learned factor (offset ``diff``), the difference set to unit RMS per
+    head and scaled by 1 - ``diff``, then gated by a sigmoid of the mixer's input.  ``chunk`` > 0:
+    a key is visible only inside the query's block of ``chunk`` positions (counted from 0)."""
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    scale: float
+    diff: float
+    rot: Optional[RotarySpec] = None
+    chunk: int = 0
+
+
+@dataclasses.dataclass(frozen=True)
+class DeltaSpec:
+    """Gated delta rule: per head a [dim, vdim] fp32 memory that decays by a data-dependent gate,
+    is corrected along the new unit key towards the new value, and is read with the unit query;
+    q, k, v pass a causal per-channel filter of ``conv`` taps and SiLU first."""
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    conv: int
+
+
+@dataclasses.dataclass(frozen=True)
+class GatedFFSpec:
+    """down(silu(gate x) * (up x))."""
+    ff: int
+
+
+@dataclasses.dataclass(frozen=True)
+class NopunexConfig:
+    """Nopunex: an fp32 residual stream with a layer norm (weight and bias) before and after every
+    sublayer; mixers are differential chunked attention, windowed latent attention with a sink, or
+    the gated delta rule; SiLU-gated dense feed-forwards (or none).  Layers ``loop[0]..loop[1]-1``
+    run ``loop[2]`` times in a row with the same weights and a cache / state per pass; every pass
+    starts from a projection of the stream joined with the embedding, plus a per-pass vector
+    (``looped`` False: no such block).  Read from a checkpoint folder's config.json
+    ("architecture": "Nopunex")."""
+    name: str
+    vocab_size: int
+    hidden_size: int
+    layers: tuple
+    rms_eps: float                  # eps of every norm of a layer
+    loop: tuple = (0, 0, 1)
+    looped: bool = False
+    logit_scale: float = 1.0
+    max_position: int = 1 << 20     # the rotation tables are built for the engine's max_model_len
+    bos_token_id: int = 0
+    eos_token_id: int = -1
+    init_std: float = 0.05
+    family: str = "nopunex"
+    is_moe: bool = False
+    experts_per_token: int = 0
+
+    @property
+    def num_layers(self) -> int:
+        return len(self.layers)
+
+    @property
+    def runs(self) -> tuple:
+        """(layer index, pass number or -1, first of its pass) of every layer run, in order."""
+        n = len(self.layers)
+        if not self.looped:
+            return tuple((i, -1, False) for i in range(n))
+        a, b, times = self.loop
+        out = [(i, -1, False) for i in range(a)]
+        for t in range(times):
+            out += [(i, t, i == a) for i in range(a, b)]
+        return tuple(out + [(i, -1, False) for i in range(b, n)])
+
+    @property
+    def needs_state(self) -> bool:
+        return any(l.type == "delta" for l in self.layers)
+
+    def num_params(self) -> int:
+        W, n = self.hidden_size, 2 * self.vocab_size * self.hidden_size
+        if self.looped:
+            n += 2 * W * W
+        for l in self.layers:
+            m = l.mixer
+            if l.type == "attention":
+                n += W * (2 * m.heads * m.dim + 2 * m.kv_heads * m.dim + m.kv_heads * m.vdim + 2 * m.heads * m.vdim)
+            elif l.type == "latent_attention":
+                n += W * (m.q_rank + m.kv_rank + m.rot_dim) + m.q_rank * m.heads * (m.dim + m.rot_dim)
+                n += m.kv_rank * m.heads * (m.dim + m.vdim) + W * m.heads * m.vdim
+            else:
+                n += W * (2 * m.kv_heads * m.dim + 3 * m.heads * m.vdim + 2 * m.heads)
+            if l.mlp is not None:
+                n += 3 * W * l.mlp.ff
+        return n
+
+    def kv_bytes_per_token(self, dtype_bytes: int = 2) -> int:
+        n = 0
+        for i, _, _ in self.runs:
+            m = self.layers[i].mixer
+            if self.layers[i].type == "attention":
+                n += m.kv_heads * (2 * m.dim + m.vdim)
+            elif self.layers[i].type == "latent_attention":
+                n += m.kv_rank + m.rot_dim
+        return n * dtype_bytes
+
+    @staticmethod
+    def _rot(r: Optional[dict]) -> Optional[RotarySpec]:
+        if not r:
+            return None
+        sc = r.get("scaling")
+        return RotarySpec(int(r["dims"]), float(r["base"]),
+                          (float(sc["factor"]), float(sc["original"]), float(sc["fast"]), float(sc["slow"])) if sc else None,
+                          halves=True)
+
+    @classmethod
+    def from_json(cls, c: dict, name: str = "nopunex") -> "NopunexConfig":
+        layers = []
+        for l in c["layers"]:
+            m = l["mixer"]
+            size = int((m.get("mask") or {}).get("size", 0))
+            if l["type"] == "attention":
+                mixer = DiffAttentionSpec(int(m["heads"]), int(m.get("kv_heads", m["heads"])), int(m["dim"]),
+                                          int(m.get("vdim", m["dim"])), float(m["scale"]), float(m["diff"]),
+                                          cls._rot(m.get("rot")), size)
+                if mixer.heads % mixer.kv_heads:
+                    raise ValueError("Nopunex: attention heads must be a multiple of kv_heads")
+            elif l["type"] == "latent_attention":
+                mixer = LatentAttentionSpec(int(m["heads"]), int(m["dim"]), int(m["vdim"]), int(m["kv_rank"]),
+                                            float(m["scale"]), int(m["q_rank"]), int(m["rot_dim"]), cls._rot(m.get("rot")),
+                                            size, True)
+                if mixer.rot is not None and mixer.rot.dims > mixer.rot_dim:
+                    raise ValueError("Nopunex: rot.dims exceeds rot_dim")
+            elif l["type"] == "delta":
+                mixer = DeltaSpec(int(m["heads"]), int(m.get("kv_heads", m["heads"])), int(m["dim"]), int(m["vdim"]),
+                                  int(m["conv"]))
+                if mixer.heads % mixer.kv_heads or mixer.conv < 1:
+                    raise ValueError("Nopunex: delta heads must be a multiple of kv_heads, conv >= 1")
+            else:
+                raise ValueError(f"Nopunex: unknown mixer type {l['type']!r}")
+            f = l.get("mlp")
+            mlp = None
+            if f is not None:
+                if f.get("kind") != "dense":
+                    raise ValueError(f"Nopunex: unknown feed-forward kind {f.get('kind')!r}")
+                mlp = GatedFFSpec(int(f["ff"]))
+            layers.append(LayerSpec(l["type"], mixer, mlp))
+        lp = c.get("loop")
+        loop = (int(lp["start"]), int(lp["stop"]), int(lp["times"])) if lp else (0, 0, 1)
+        if not (0 <= loop[0] <= loop[1] <= len(layers)) or loop[2] < 1:
+            raise ValueError(f"Nopunex: loop {loop} does not fit {len(layers)} layers")
+        return cls(name=name, vocab_size=int(c["vocab"]), hidden_size=int(c["width"]), layers=tuple(layers),
+                   rms_eps=float(c["norm"]["eps"]), loop=loop, looped=bool(lp) and loop[1] > loop[0],
+                   logit_scale=float(c.get("logit_scale", 1.0)))
+
+    @classmethod
+    def uniform(cls, name: str, vocab: int, width: int, pattern: str, heads: int, kv_heads: int, dim: int, ff: int,
+                kv_rank: int = 512, q_rank: int = 1024, rot_dim: int = 64, window: int = 1024, chunk: int = 1024,
+                loop: Optional[tuple] = None) -> "NopunexConfig":
+        """``pattern``: one letter per layer, A differential attention / M latent attention /
+        D delta rule; lower case: without a feed-forward."""
+        layers = []
+        for ch in pattern:
+            up = ch.upper()
+            if up == "A":
+                mixer = DiffAttentionSpec(heads, kv_heads, dim, dim, dim ** -0.5, 0.3,
+                                          RotarySpec(dim // 2, 1e6, None, True), chunk)
+            elif up == "M":
+                mixer = LatentAttentionSpec(heads, dim, dim, kv_rank, (dim + rot_dim) ** -0.5, q_rank, rot_dim,
+                                            RotarySpec(rot_dim, 5e5, (8.0, 4096.0, 32.0, 1.0), True), window, True)
+            else:
+                mixer = DeltaSpec(heads, kv_heads, dim, dim, 4)
+            layers.append(LayerSpec({"A": "attention", "M": "latent_attention", "D": "delta"}[up], mixer,
+                                    GatedFFSpec(ff) if ch.isupper() else None))
+        return cls(name=name, vocab_size=vocab, hidden_size=width, layers=tuple(layers), rms_eps=1e-5,
+                   loop=loop or (0, 0, 1), looped=loop is not None, logit_scale=1.0)
+
+
 # config.json "architecture" -> reader (checkpoints that are not HF Llama / Mixtral folders)
-ARCHITECTURES = {"Sapapel": SapapelConfig.from_json, "Kivezen": KivezenConfig.from_json}
+ARCHITECTURES = {"Sapapel": SapapelConfig.from_json, "Kivezen": KivezenConfig.from_json,
+                 "Nopunex": NopunexConfig.from_json}
 
 PRESETS["tiny-sapapel"] = SapapelConfig.uniform("tiny-sapapel", 512, 128, 3, 4, 16, 32, 48, 64, 6, 2)
 # speed measurements (random weights): layer shapes of small production MoE models, and the
@@ -362,6 +552,15 @@ PRESETS["tiny-kivezen"] = KivezenConfig.uniform("tiny-kivezen", 512, 128, "LAa",
 # and expert size; every fourth mixer is a lightning layer, every layer has the MoE with a shared expert
 PRESETS["kivezen-2k"] = KivezenConfig.uniform("kivezen-2k", 32000, 2048, "LAAALAAA", 16, 4, 128, 4096, 16, 2, 1536)
 PRESETS["kivezen-4k"] = KivezenConfig.uniform("kivezen-4k", 32000, 4096, "LAAA", 32, 8, 128, 8192, 8, 2, 2048)
+
+
+PRESETS["tiny-nopunex"] = NopunexConfig.uniform("tiny-nopunex", 512, 128, "AdMA", 4, 2, 32, 256, kv_rank=48, q_rank=64,
+                                                rot_dim=16, window=40, chunk=24, loop=(1, 3, 2))
+# speed measurements beside kivezen-2k / kivezen-4k (the closest family: fp32 stream, a recurrent
+# mixer among attention layers): the same width, depth, heads, KV heads and head size, dense
+# feed-forwards of the MoE's active size
+PRESETS["nopunex-2k"] = NopunexConfig.uniform("nopunex-2k", 32000, 2048, "DAMADAMA", 16, 4, 128, 4608)
+PRESETS["nopunex-4k"] = NopunexConfig.uniform("nopunex-4k", 32000, 4096, "DAMA", 32, 8, 128, 6144)
 
 
 def get_config(name_or_path: str):
