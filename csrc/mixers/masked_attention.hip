@@ -1,0 +1,467 @@
+// Softmax attention over a paged cache with a band of visible keys per query, learned sinks and
+// separate counts of query, key and value heads; the rotations and cache writes in front of it; and
+// the per-head norm / gate behind it.
+//
+//   rotate_cache      q and k heads turn by the token's position (fp32 (cos, sin) table rows; pair i
+//                     = (i, i + pairs) or (2i, 2i + 1)); q -> [T, QH, D], k -> cache
+//                     [blocks, KH, block_size, D], v -> cache [blocks, VH, block_size, V]
+//   latent_in         a projection row [query latent | key / value latent | shared key part]: both
+//                     latents set to unit RMS times a weight, the key part turned by the position;
+//                     the query latent is returned, [latent | key part] goes to the cache row
+//   latent_query      [folded query | the head's rotated part turned by the position] in fp32
+//   masked_attention  query at position p sees keys lo(p) <= j <= p, lo(p) = max(0, p - window + 1,
+//                     floor(p / chunk) chunk); p_j = exp(s_j) / (exp(sink_h) + sum_j' exp(s_j')),
+//                     s = q . k * scale; o = sum_j p_j v_j.  Query head h reads key head h / (QH / KH)
+//                     and value head h / (QH / VH); the value may be the first V numbers of the key row.
+//   head_norm_gate    per (token, head): u / sqrt(mean(u^2) + eps) * w * post * act(gate), with u one
+//                     head's row or the difference first - coef * second of two attention maps
+//
+// Scores, softmax, sums and norms are fp32 for both element types.  The (token, head) pairs of a
+// sequence that share a key head are the rows of one tile problem against key / value tiles staged
+// once in LDS; key tiles start at multiples of the tile size counted from key 0 of the sequence, so
+// a position's sums run in the same order however its prompt was cut and whatever else the step holds.
+#include "mix_common.h"
+
+using namespace pkm;
+
+namespace {
+
+__device__ __forceinline__ int clamp_pos(int pos, int rows) { return pos < 0 ? 0 : (pos >= rows ? max(rows - 1, 0) : pos); }
+
+// one wave turns one head: x[i], x[i + pairs] (halves) or x[2i], x[2i + 1] of the first 2 * pairs
+// coordinates by (cos, sin) = cs[2i], cs[2i + 1]; the rest pass.  IN -> OUT element types.
+template <typename IN, typename OUT>
+__device__ __forceinline__ void turn_head(OUT* dst, const IN* src, int D, const float* cs, int pairs, int halves, int lane) {
+  for (int i = lane; i < pairs; i += 64) {
+    const int iu = halves ? i : 2 * i, iv = halves ? i + pairs : 2 * i + 1;
+    const float u = ld<IN>(src + iu), v = ld<IN>(src + iv);
+    const float c = cs[2 * i], s = cs[2 * i + 1];
+    st<OUT>(dst + iu, u * c - v * s);
+    st<OUT>(dst + iv, v * c + u * s);
+  }
+  for (int i = 2 * pairs + lane; i < D; i += 64) st<OUT>(dst + i, ld<IN>(src + i));
+}
+
+template <typename T>
+__global__ void __launch_bounds__(64)
+rotate_cache_kernel(T* __restrict__ q_out, const T* __restrict__ proj, int64_t stride, const int* __restrict__ positions,
+                    const int* __restrict__ slot_mapping, const float* __restrict__ table, int pairs, int table_rows,
+                    int halves, T* __restrict__ k_cache, T* __restrict__ v_cache, int QH, int KH, int VH, int D, int V,
+                    int bs) {
+  const int t = blockIdx.x, item = blockIdx.y, lane = threadIdx.x;
+  const int slot = slot_mapping[t];
+  const T* row = proj + static_cast<int64_t>(t) * stride;
+  const float* cs = table ? table + static_cast<int64_t>(clamp_pos(positions[t], table_rows)) * pairs * 2 : nullptr;
+  const int np = cs ? pairs : 0;
+  if (item < QH) {
+    turn_head<T, T>(q_out + (static_cast<int64_t>(t) * QH + item) * D, row + static_cast<int64_t>(item) * D, D, cs, np,
+                    halves, lane);
+  } else if (item < QH + KH) {
+    if (slot < 0) return;
+    const int g = item - QH;
+    turn_head<T, T>(k_cache + ((static_cast<int64_t>(slot / bs) * KH + g) * bs + slot % bs) * D,
+                    row + static_cast<int64_t>(item) * D, D, cs, np, halves, lane);
+  } else {
+    if (slot < 0) return;
+    const int g = item - QH - KH;
+    const T* src = row + static_cast<int64_t>(QH + KH) * D + static_cast<int64_t>(g) * V;
+    T* dst = v_cache + ((static_cast<int64_t>(slot / bs) * VH + g) * bs + slot % bs) * V;
+    for (int i = lane; i < V; i += 64) dst[i] = src[i];
+  }
+}
+
+// blockIdx.y: 0 the query latent, 1 the key / value latent and the shared key part
+template <typename T>
+__global__ void __launch_bounds__(256)
+latent_in_kernel(T* __restrict__ cq, T* __restrict__ cache, const T* __restrict__ proj, int64_t stride, int Q, int R, int Dr,
+                 const float* __restrict__ wq, const float* __restrict__ wkv, float eps, const int* __restrict__ positions,
+                 const int* __restrict__ slot_mapping, const float* __restrict__ table, int pairs, int table_rows,
+                 int halves, int bs) {
+  __shared__ float red[16];
+  const int t = blockIdx.x, tid = threadIdx.x;
+  const T* row = proj + static_cast<int64_t>(t) * stride;
+  const bool query = blockIdx.y == 0;
+  if (query && Q == 0) return;
+  const int slot = slot_mapping[t];
+  if (!query && slot < 0) return;
+  const T* src = query ? row : row + Q;
+  const int n = query ? Q : R;
+  const float* w = query ? wq : wkv;
+  T* dst = query ? cq + static_cast<int64_t>(t) * Q : cache + static_cast<int64_t>(slot) * (R + Dr);
+  float ss = 0.f;
+  for (int i = tid; i < n; i += 256) {
+    const float v = ld<T>(src + i);
+    ss += v * v;
+  }
+  ss = pk::block_sum(ss, red);
+  const float k = 1.f / sqrtf(ss / static_cast<float>(n) + eps);
+  for (int i = tid; i < n; i += 256) st<T>(dst + i, ld<T>(src + i) * k * w[i]);
+  if (!query && tid < 64 && Dr > 0) {
+    const float* cs = table ? table + static_cast<int64_t>(clamp_pos(positions[t], table_rows)) * pairs * 2 : nullptr;
+    turn_head<T, T>(dst + R, src + R, Dr, cs, cs ? pairs : 0, halves, tid);
+  }
+}
+
+template <typename T>
+__global__ void __launch_bounds__(64)
+latent_query_kernel(float* __restrict__ out, const T* __restrict__ q_lat, const T* __restrict__ q,
+                    const int* __restrict__ positions, const float* __restrict__ table, int pairs, int table_rows,
+                    int halves, int T_, int H, int R, int D, int Dr) {
+  const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  float* dst = out + (static_cast<int64_t>(t) * H + h) * (R + Dr);
+  const T* src = q_lat + (static_cast<int64_t>(h) * T_ + t) * R;
+  for (int i = lane; i < R; i += 64) dst[i] = ld<T>(src + i);
+  if (Dr > 0) {
+    const float* cs = table ? table + static_cast<int64_t>(clamp_pos(positions[t], table_rows)) * pairs * 2 : nullptr;
+    turn_head<T, float>(dst + R, q + (static_cast<int64_t>(t) * H + h) * (D + Dr) + D, Dr, cs, cs ? pairs : 0, halves, lane);
+  }
+}
+
+constexpr int kBQ = 16;        // (token, head) rows per workgroup
+constexpr int kThreads = 256;  // 16 rows x 16 lanes
+
+struct MaskedArgs {
+  void* out;
+  int64_t out_ts, out_hs;  // element strides of a token and of a head in out
+  int out_f32;
+  const void* q;  // [T, QH, D]
+  int q_f32;
+  const void* k_cache;  // [blocks, KH, bs, D]
+  const void* v_cache;  // [blocks, VH, bs, v_width]
+  int v_width;
+  const int* block_tables;
+  int64_t bt_stride;
+  const int* cu_q;
+  const int* context_lens;
+  const float* sink;  // [QH] logits or null
+  int n_seqs, QH, KH, VH, D, V, bs, BK;
+  float scale;
+  int window, chunk;
+};
+
+__device__ __forceinline__ int first_key(int pos, int window, int chunk) {
+  int lo = 0;
+  if (window > 0) lo = max(lo, pos - window + 1);
+  if (chunk > 0) lo = max(lo, pos / chunk * chunk);
+  return lo;
+}
+
+// NV: output accumulators per thread = ceil(V / 16).  ALIAS: the value of a key is the first V
+// numbers of its key row (KH == VH, same cache).
+template <typename T, int NV, bool ALIAS>
+__global__ void __launch_bounds__(kThreads) masked_attention_kernel(MaskedArgs a) {
+  extern __shared__ float smem[];
+  const int QH = a.QH, KH = a.KH, D = a.D, V = a.V, BK = a.BK, bs = a.bs;
+  const int R = QH / KH;  // query heads per key head
+  const int kh = blockIdx.y;
+  const int vh = kh / (KH / a.VH);
+  int s = 0, tile = blockIdx.x;
+  for (; s < a.n_seqs; ++s) {
+    const int rows = (a.cu_q[s + 1] - a.cu_q[s]) * R;
+    const int nt = (rows + kBQ - 1) / kBQ;
+    if (tile < nt) break;
+    tile -= nt;
+  }
+  if (s >= a.n_seqs) return;
+  const int q0 = a.cu_q[s], qlen = a.cu_q[s + 1] - q0, ctx = a.context_lens[s];
+  const int n_rows = qlen * R;
+  const int row0 = tile * kBQ;
+  const int DS = D + 1, VS = V + 1;  // odd row strides: conflict-free column walks
+  float* qs = smem;                  // [kBQ][DS]
+  float* ks = qs + kBQ * DS;         // [BK][DS]
+  float* vs = ALIAS ? ks : ks + BK * DS;           // [BK][VS] (ALIAS: the key rows)
+  float* ps = ALIAS ? ks + BK * DS : vs + BK * VS;  // [kBQ][BK]
+  float* m_s = ps + kBQ * BK;        // [kBQ] running max
+  float* l_s = m_s + kBQ;            // [kBQ] running sum
+  const int vstride = ALIAS ? DS : VS;
+  const int tid = threadIdx.x;
+  const int qi = tid >> 4, kg = tid & 15;
+  const int* bt = a.block_tables + static_cast<int64_t>(s) * a.bt_stride;
+  const T* kc = static_cast<const T*>(a.k_cache);
+  const T* vc = static_cast<const T*>(a.v_cache);
+
+  for (int e = tid; e < kBQ * D; e += kThreads) {
+    const int r = e / D, c = e - r * D;
+    const int row = row0 + r;
+    float v = 0.f;
+    if (row < n_rows) {
+      const int tl = row / R, h = kh * R + row - tl * R;
+      const int64_t at = (static_cast<int64_t>(q0 + tl) * QH + h) * D + c;
+      v = a.q_f32 ? static_cast<const float*>(a.q)[at] : ld<T>(static_cast<const T*>(a.q) + at);
+    }
+    qs[r * DS + c] = v;
+  }
+  const int my_row = row0 + qi;
+  const bool live = my_row < n_rows;
+  const int my_tl = live ? my_row / R : 0;
+  const int my_h = kh * R + (live ? my_row - my_tl * R : 0);
+  const int my_pos = live ? ctx - qlen + my_tl : -1;
+  const int my_lo = live ? first_key(my_pos, a.window, a.chunk) : 0;
+  if (tid < kBQ) {
+    const int row = row0 + tid;
+    const int h = kh * R + (row < n_rows ? row % R : 0);
+    m_s[tid] = a.sink ? a.sink[h] : -INFINITY;  // the sink is a key without a value
+    l_s[tid] = a.sink ? 1.f : 0.f;
+  }
+  const int first_pos = ctx - qlen + row0 / R;
+  const int last_pos = ctx - qlen + (min(row0 + kBQ, n_rows) - 1) / R;
+  const int k_end = last_pos + 1;  // keys [k_begin, k_end) are visible to some row
+  const int k_begin = first_pos >= 0 ? first_key(first_pos, a.window, a.chunk) / BK * BK : 0;
+  float acc[NV];
+#pragma unroll
+  for (int i = 0; i < NV; ++i) acc[i] = 0.f;
+  __syncthreads();
+
+  for (int k0 = k_begin; k0 < k_end; k0 += BK) {
+    const int nk = min(BK, k_end - k0);
+    for (int e = tid; e < BK * D; e += kThreads) {
+      const int j = e / D, c = e - j * D;
+      float v = 0.f;
+      if (j < nk) {
+        const int key = k0 + j;
+        v = ld<T>(kc + ((static_cast<int64_t>(bt[key / bs]) * KH + kh) * bs + key % bs) * D + c);
+      }
+      ks[j * DS + c] = v;
+    }
+    if (!ALIAS) {
+      for (int e = tid; e < BK * V; e += kThreads) {
+        const int j = e / V, c = e - j * V;
+        float v = 0.f;
+        if (j < nk) {
+          const int key = k0 + j;
+          v = ld<T>(vc + ((static_cast<int64_t>(bt[key / bs]) * a.VH + vh) * bs + key % bs) * a.v_width + c);
+        }
+        vs[j * VS + c] = v;
+      }
+    }
+    __syncthreads();
+    float tmax = -INFINITY;
+    for (int j = kg; j < BK; j += 16) {
+      float d = 0.f;
+      const float* qr = qs + qi * DS;
+      const float* kr = ks + j * DS;
+      for (int c = 0; c < D; ++c) d += qr[c] * kr[c];
+      d *= a.scale;
+      const int key = k0 + j;
+      d = (j < nk && key <= my_pos && key >= my_lo) ? d : -INFINITY;
+      ps[qi * BK + j] = d;
+      tmax = fmaxf(tmax, d);
+    }
+#pragma unroll
+    for (int o = 8; o > 0; o >>= 1) tmax = fmaxf(tmax, __shfl_xor(tmax, o, 64));
+    const float m_old = m_s[qi];
+    const float m_new = fmaxf(m_old, tmax);
+    float tsum = 0.f;
+    for (int j = kg; j < BK; j += 16) {
+      const float sc = ps[qi * BK + j];
+      const float p = (m_new == -INFINITY || sc == -INFINITY) ? 0.f : expf(sc - m_new);
+      ps[qi * BK + j] = p;
+      tsum += p;
+    }
+#pragma unroll
+    for (int o = 8; o > 0; o >>= 1) tsum += __shfl_xor(tsum, o, 64);
+    const float resc = (m_old == -INFINITY) ? 0.f : expf(m_old - m_new);
+    __syncthreads();  // every lane of the row has read m_old and its own scores
+    if (kg == 0) {
+      m_s[qi] = m_new;
+      l_s[qi] = l_s[qi] * resc + tsum;
+    }
+#pragma unroll
+    for (int i = 0; i < NV; ++i) acc[i] *= resc;
+    for (int j = 0; j < nk; ++j) {
+      const float p = ps[qi * BK + j];
+      const float* vr = vs + j * vstride + kg;
+#pragma unroll
+      for (int i = 0; i < NV; ++i)
+        if (kg + 16 * i < V) acc[i] += p * vr[16 * i];
+    }
+    __syncthreads();
+  }
+  const float l = l_s[qi];
+  const float inv = l > 0.f ? 1.f / l : 0.f;
+  if (!live) return;
+  const int64_t at = static_cast<int64_t>(q0 + my_tl) * a.out_ts + static_cast<int64_t>(my_h) * a.out_hs;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int c = kg + 16 * i;
+    if (c < V) {
+      if (a.out_f32) {
+        static_cast<float*>(a.out)[at + c] = acc[i] * inv;
+      } else {
+        st<T>(static_cast<T*>(a.out) + at + c, acc[i] * inv);
+      }
+    }
+  }
+}
+
+size_t lds_bytes(int D, int V, int bk, bool alias) {
+  return (static_cast<size_t>(kBQ) * (D + 1) + static_cast<size_t>(bk) * (D + 1 + (alias ? 0 : V + 1)) + kBQ * bk + 2 * kBQ) * 4;
+}
+
+// key tile: the largest of 64 / 32 / 16 whose tiles fit 60 KiB of LDS, else the largest of 32 / 16 / 8
+// within 144 KiB; 0: the heads are too wide
+int key_tile(int D, int V, bool alias) {
+  for (int bk = 64; bk >= 16; bk >>= 1)
+    if (lds_bytes(D, V, bk, alias) <= 60 * 1024) return bk;
+  for (int bk = 32; bk >= 8; bk >>= 1)
+    if (lds_bytes(D, V, bk, alias) <= 144 * 1024) return bk;
+  return 0;
+}
+
+template <typename T, int NV, bool ALIAS>
+int launch_one(const MaskedArgs& a, dim3 grid, size_t lds, hipStream_t stream) {
+  if (lds > 60 * 1024) {
+    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(masked_attention_kernel<T, NV, ALIAS>),
+                                             hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
+    if (e != hipSuccess) return static_cast<int>(e);
+  }
+  masked_attention_kernel<T, NV, ALIAS><<<grid, kThreads, lds, stream>>>(a);
+  return PK_CHECK_LAUNCH();
+}
+
+template <typename T, bool ALIAS>
+int launch_masked(const MaskedArgs& a, dim3 grid, hipStream_t stream) {
+  const size_t lds = lds_bytes(a.D, a.V, a.BK, ALIAS);
+  const int nv = (a.V + 15) / 16;
+  if (nv <= 1) return launch_one<T, 1, ALIAS>(a, grid, lds, stream);
+  if (nv <= 2) return launch_one<T, 2, ALIAS>(a, grid, lds, stream);
+  if (nv <= 4) return launch_one<T, 4, ALIAS>(a, grid, lds, stream);
+  if (nv <= 8) return launch_one<T, 8, ALIAS>(a, grid, lds, stream);
+  if (nv <= 16) return launch_one<T, 16, ALIAS>(a, grid, lds, stream);
+  return launch_one<T, 32, ALIAS>(a, grid, lds, stream);
+}
+
+constexpr int kGateNone = 0, kGateSigmoid = 1, kGateSilu = 2;
+
+// one wave per (token, head)
+template <typename GT, typename OT>
+__global__ void __launch_bounds__(64)
+head_norm_gate_kernel(OT* __restrict__ out, const float* __restrict__ a, int H, int V, float eps, const GT* __restrict__ gate,
+                      int64_t gate_stride, int gate_kind, const float* __restrict__ weight, float post, int pair_group,
+                      float coef) {
+  const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const float *u1, *u2 = nullptr;
+  if (pair_group > 0) {
+    const int g = h / pair_group, j = h - g * pair_group;
+    u1 = a + (static_cast<int64_t>(t) * 2 * H + static_cast<int64_t>(g) * 2 * pair_group + j) * V;
+    u2 = u1 + static_cast<int64_t>(pair_group) * V;
+  } else {
+    u1 = a + (static_cast<int64_t>(t) * H + h) * V;
+  }
+  float ss = 0.f;
+  for (int i = lane; i < V; i += 64) {
+    const float u = u2 ? u1[i] - coef * u2[i] : u1[i];
+    ss += u * u;
+  }
+  ss = pk::wave_sum(ss);
+  const float k = post / sqrtf(ss / static_cast<float>(V) + eps);
+  OT* dst = out + (static_cast<int64_t>(t) * H + h) * V;
+  const GT* gr = gate ? gate + static_cast<int64_t>(t) * gate_stride + static_cast<int64_t>(h) * V : nullptr;
+  for (int i = lane; i < V; i += 64) {
+    float z = (u2 ? u1[i] - coef * u2[i] : u1[i]) * k;
+    if (weight) z *= weight[i];
+    if (gr && gate_kind != kGateNone) {
+      const float g = ld<GT>(gr + i);
+      z *= gate_kind == kGateSigmoid ? sigmoidf(g) : g * sigmoidf(g);
+    }
+    st<OT>(dst + i, z);
+  }
+}
+
+}  // namespace
+
+// proj [T, QH*D | KH*D | VH*V] rows `stride` elements apart; table [table_rows, pairs, 2] fp32 or null
+PK_EXPORT int pkm_rotate_cache(void* q_out, const void* proj, long long stride, const void* positions,
+                               const void* slot_mapping, const void* table, int pairs, int table_rows, int halves,
+                               void* k_cache, void* v_cache, int T, int QH, int KH, int VH, int D, int V, int bs, int dt,
+                               hipStream_t stream) {
+  if (T <= 0) return 0;
+  if (D < 1 || V < 1 || 2 * pairs > D || (table && table_rows < 1) || bs < 1) return -1;
+  const dim3 grid(T, QH + KH + VH);
+  PKM_DISPATCH(dt, E, rotate_cache_kernel<E><<<grid, 64, 0, stream>>>(
+                          static_cast<E*>(q_out), static_cast<const E*>(proj), stride, static_cast<const int*>(positions),
+                          static_cast<const int*>(slot_mapping), static_cast<const float*>(table), pairs, table_rows,
+                          halves, static_cast<E*>(k_cache), static_cast<E*>(v_cache), QH, KH, VH, D, V, bs));
+  return PK_CHECK_LAUNCH();
+}
+
+// proj [T, Q | R | Dr]; cq [T, Q] (null with Q = 0); cache rows [slots, R + Dr]
+PK_EXPORT int pkm_latent_in(void* cq, void* cache, const void* proj, long long stride, int Q, int R, int Dr, const void* wq,
+                            const void* wkv, float eps, const void* positions, const void* slot_mapping,
+                            const void* table, int pairs, int table_rows, int halves, int T, int bs, int dt,
+                            hipStream_t stream) {
+  if (T <= 0) return 0;
+  if (R < 1 || Q < 0 || Dr < 0 || 2 * pairs > Dr || (table && table_rows < 1) || (Q > 0 && (!cq || !wq))) return -1;
+  const dim3 grid(T, 2);
+  PKM_DISPATCH(dt, E, latent_in_kernel<E><<<grid, 256, 0, stream>>>(
+                          static_cast<E*>(cq), static_cast<E*>(cache), static_cast<const E*>(proj), stride, Q, R, Dr,
+                          static_cast<const float*>(wq), static_cast<const float*>(wkv), eps,
+                          static_cast<const int*>(positions), static_cast<const int*>(slot_mapping),
+                          static_cast<const float*>(table), pairs, table_rows, halves, bs));
+  return PK_CHECK_LAUNCH();
+}
+
+// out [T, H, R + Dr] fp32; q_lat [H, T, R]; q [T, H, D + Dr]
+PK_EXPORT int pkm_latent_query(void* out, const void* q_lat, const void* q, const void* positions, const void* table,
+                               int pairs, int table_rows, int halves, int T, int H, int R, int D, int Dr, int dt,
+                               hipStream_t stream) {
+  if (T <= 0) return 0;
+  if (2 * pairs > Dr || (table && table_rows < 1)) return -1;
+  const dim3 grid(T, H);
+  PKM_DISPATCH(dt, E, latent_query_kernel<E><<<grid, 64, 0, stream>>>(
+                          static_cast<float*>(out), static_cast<const E*>(q_lat), static_cast<const E*>(q),
+                          static_cast<const int*>(positions), static_cast<const float*>(table), pairs, table_rows, halves,
+                          T, H, R, D, Dr));
+  return PK_CHECK_LAUNCH();
+}
+
+// v_cache == k_cache: the value of a key is the first V numbers of its key row
+PK_EXPORT int pkm_masked_attention(void* out, long long out_ts, long long out_hs, int out_dt, const void* q, int q_dt,
+                                   const void* k_cache, const void* v_cache, int v_width, const void* block_tables,
+                                   long long bt_stride, const void* cu_q, const void* context_lens, const void* sink,
+                                   int n_seqs, int T, int QH, int KH, int VH, int D, int V, int bs, float scale, int window,
+                                   int chunk, int dt, hipStream_t stream) {
+  if (n_seqs <= 0 || T <= 0) return 0;
+  if (KH < 1 || VH < 1 || QH % KH || KH % VH || V < 1 || V > 512 || V > v_width || D < 1) return -1;
+  if ((q_dt != dt && q_dt != kF32) || (out_dt != dt && out_dt != kF32)) return -1;
+  const bool alias = v_cache == k_cache;
+  if (alias && (KH != VH || v_width != D)) return -1;
+  const int bk = key_tile(D, V, alias);
+  if (bk == 0) return -1;
+  MaskedArgs a{out, out_ts, out_hs, out_dt == kF32, q, q_dt == kF32, k_cache, v_cache, v_width,
+               static_cast<const int*>(block_tables), bt_stride, static_cast<const int*>(cu_q),
+               static_cast<const int*>(context_lens), static_cast<const float*>(sink), n_seqs, QH, KH, VH, D, V, bs, bk,
+               scale, window, chunk};
+  const int R = QH / KH;
+  // row tiles: every sequence adds at most one partly filled tile
+  const int tiles = (T * R + kBQ - 1) / kBQ + n_seqs;
+  const dim3 grid(tiles, KH);
+  if (alias) {
+    PKM_DISPATCH(dt, E, return (launch_masked<E, true>(a, grid, stream)));
+  }
+  PKM_DISPATCH(dt, E, return (launch_masked<E, false>(a, grid, stream)));
+  return 0;
+}
+
+// a fp32 [T, H, V] (pair_group = 0) or [T, 2H, V] in groups of (r first maps, r second maps);
+// gate [T, H * V] rows gate_stride elements apart (gate_dt) or null; weight [V] fp32 or null
+PK_EXPORT int pkm_head_norm_gate(void* out, const void* a, int T, int H, int V, float eps, const void* gate,
+                                 long long gate_stride, int gate_dt, int gate_kind, const void* weight, float post,
+                                 int pair_group, float coef, int out_dt, hipStream_t stream) {
+  if (T <= 0) return 0;
+  if (H < 1 || V < 1 || pair_group < 0 || (pair_group > 0 && H % pair_group)) return -1;
+  const dim3 grid(T, H);
+#define PKM_HNG(GT)                                                                                                  \
+  PKM_DISPATCH(out_dt, O, head_norm_gate_kernel<GT, O><<<grid, 64, 0, stream>>>(                                       \
+                              static_cast<O*>(out), static_cast<const float*>(a), H, V, eps, static_cast<const GT*>(gate), \
+                              gate_stride, gate_kind, static_cast<const float*>(weight), post, pair_group, coef))
+  if (gate_dt == kF32) {
+    PKM_HNG(float);
+  } else if (gate_dt == kBF16) {
+    PKM_HNG(bf16_t);
+  } else {
+    return -2;
+  }
+#undef PKM_HNG
+  return PK_CHECK_LAUNCH();
+}

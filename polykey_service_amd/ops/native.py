@@ -100,6 +100,18 @@ MIXER_SIGNATURES = {
     "pkm_rope_norm_cache": [P, P, I64, I32, P, P, P, I32, P, I32, P, P, I32, I32, I32, I32, I32, I32, F32, I32, P],
     "pkm_sink_decode_part": [I32, I32, I32, I32, I32],
     "pkm_set_sink_mfma": [I32],
+    "pkm_sandwich_step": [P, I32, I32, P, I32, I32, P, P, I32, P, P, P, F32, P, I32, P, P],
+    "pkm_join_cast": [P, P, P, I32, I32, I32, P],
+    "pkm_silu_mul": [P, P, I32, I32, I32, I32, I32, P],
+    "pkm_scale": [P, I64, F32, P],
+    "pkm_rotate_cache": [P, P, I64, P, P, P, I32, I32, I32, P, P, I32, I32, I32, I32, I32, I32, I32, I32, P],
+    "pkm_latent_in": [P, P, P, I64, I32, I32, I32, P, P, F32, P, P, P, I32, I32, I32, I32, I32, I32, P],
+    "pkm_latent_query": [P, P, P, P, P, I32, I32, I32, I32, I32, I32, I32, I32, I32, P],
+    "pkm_masked_attention": [P, I64, I64, I32, P, I32, P, P, I32, P, I64, P, P, P, I32, I32, I32, I32, I32, I32, I32, I32,
+                             F32, I32, I32, I32, P],
+    "pkm_head_norm_gate": [P, P, I32, I32, I32, F32, P, I64, I32, I32, P, F32, I32, F32, I32, P],
+    "pkm_conv_unit": [P, P, I64, P, I32, P, P, P, P, P, I32, I32, I32, I32, I32, I32, I32, P],
+    "pkm_delta_rule": [P, P, P, I64, I32, P, P, P, P, P, P, I32, I32, I32, I32, I32, I32, P],
     "pkm_sink_attention": [P, P, P, P, P, I64, P, P, P, P, P, I32, I32, I32, I32, I32, I32, I32, I32, F32, F32, I32,
                            P, P, I32, I32, I32, P],
 }

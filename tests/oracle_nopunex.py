@@ -200,3 +200,75 @@ def forward(cfg: dict, w: Dict[str, torch.Tensor], tokens, layers_out: Optional[
             layers_out.append(x)
     x = layer_norm(x, w["final.norm"], w["final.norm.b"], eps)
     return (x @ w["head"].T) * float(cfg.get("logit_scale", 1.0))
+
+
+# ------------------------------------------------------- configurations and weights for tests
+def make_config(vocab=80, width=48, pattern="AdMA", heads=4, kv_heads=2, dim=8, vdim=12, rot_dims=6, ff=40, chunk=16,
+                window=24, kv_rank=20, q_rank=28, rot_dim=6, conv=3, loop=None, diff=0.3, scaling=(4.0, 64, 8.0, 1.0),
+                logit_scale=1.5, eps=1e-5) -> dict:
+    """``pattern``: A differential attention / M latent attention / D delta rule per layer, lower
+    case without a feed-forward."""
+    layers = []
+    for ch in pattern:
+        up = ch.upper()
+        if up == "A":
+            m = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": dim ** -0.5, "diff": diff,
+                 "mask": {"size": chunk}, "rot": {"dims": rot_dims, "base": 10000.0}}
+            if not rot_dims:
+                del m["rot"]
+        elif up == "M":
+            rot = {"dims": rot_dim, "base": 5000.0}
+            if scaling:
+                rot["scaling"] = dict(zip(("factor", "original", "fast", "slow"), scaling))
+            m = {"heads": heads, "dim": dim, "rot_dim": rot_dim, "vdim": vdim, "kv_rank": kv_rank, "q_rank": q_rank,
+                 "scale": (dim + rot_dim) ** -0.5, "mask": {"size": window}, "rot": rot}
+        else:
+            m = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "conv": conv}
+        layers.append({"type": {"A": "attention", "M": "latent_attention", "D": "delta"}[up], "mixer": m,
+                       "mlp": {"kind": "dense", "ff": ff} if ch.isupper() else None})
+    cfg = {"architecture": "Nopunex", "vocab": vocab, "width": width, "layers": layers, "norm": {"eps": eps},
+           "logit_scale": logit_scale}
+    if loop:
+        cfg["loop"] = dict(zip(("start", "stop", "times"), loop))
+    return cfg
+
+
+def random_model(cfg: dict, seed: int = 0, std: float = 0.25) -> Dict[str, torch.Tensor]:
+    """bf16-representable random tensors under the checkpoint names."""
+    g = torch.Generator().manual_seed(seed)
+    W = cfg["width"]
+    r = lambda *shape, s=std: (torch.randn(*shape, generator=g) * s).bfloat16().double()
+    w = {"embed": r(cfg["vocab"], W, s=1.0), "head": r(cfg["vocab"], W)}
+
+    def norm(name):
+        w[name], w[name + ".b"] = (1 + r(W, s=0.1)).bfloat16().double(), r(W, s=0.1)
+    norm("final.norm")
+    if cfg.get("loop"):
+        w["loop.in"] = r(W, 2 * W, s=(2 * W) ** -0.5)
+        w["loop.step"] = r(cfg["loop"]["times"], W, s=0.2)
+    for i, l in enumerate(cfg["layers"]):
+        p, m = f"l{i}.", l["mixer"]
+        for q in ["1", "1b"] + (["2", "2b"] if l["mlp"] else []):
+            norm(p + "norm" + q)
+        p += "mix."
+        if l["type"] == "attention":
+            H, G, D, V = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+            w.update({p + "q": r(2 * H * D, W), p + "k": r(2 * G * D, W), p + "v": r(G * V, W), p + "g": r(H * V, W),
+                      p + "o": r(W, H * V)})
+            for n in ("lq1", "lk1", "lq2", "lk2"):
+                w[p + n] = r(D, s=0.3)
+        elif l["type"] == "latent_attention":
+            H, D, Dr, V, R, Q = m["heads"], m["dim"], m["rot_dim"], m["vdim"], m["kv_rank"], m["q_rank"]
+            w.update({p + "dq": r(Q, W), p + "dq.norm": (1 + r(Q, s=0.1)).bfloat16().double(), p + "uq": r(H * (D + Dr), Q),
+                      p + "dkv": r(R + Dr, W), p + "dkv.norm": (1 + r(R, s=0.1)).bfloat16().double(),
+                      p + "uk": r(H * D, R), p + "uv": r(H * V, R), p + "sink": r(H, s=1.0), p + "o": r(W, H * V)})
+        else:
+            H, G, D, V, K = m["heads"], m["kv_heads"], m["dim"], m["vdim"], m["conv"]
+            w.update({p + "q": r(G * D, W), p + "k": r(G * D, W), p + "v": r(H * V, W), p + "a": r(H, W), p + "b": r(H, W),
+                      p + "g": r(H * V, W), p + "o": r(W, H * V), p + "q.conv": r(G * D, K, s=0.6),
+                      p + "k.conv": r(G * D, K, s=0.6), p + "v.conv": r(H * V, K, s=0.6), p + "A_log": r(H, s=0.7),
+                      p + "dt_bias": r(H, s=0.7), p + "norm": (1 + r(V, s=0.1)).bfloat16().double()})
+        if l["mlp"]:
+            F = l["mlp"]["ff"]
+            w.update({f"l{i}.mlp.gate": r(F, W), f"l{i}.mlp.up": r(F, W), f"l{i}.mlp.down": r(W, F)})
+    return w
