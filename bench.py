@@ -101,10 +101,13 @@ def parse_args(argv=None):
                          "JSON line is always printed in time")
     ap.add_argument("--compare-families", default="",
                     help="instead of the headline workload: engine-level prefill and decode throughput of the "
-                         "--compare-family family beside the Mixtral family at equal layer sizes, e.g. '2k,4k' "
-                         "(presets <family>-<size> / mixtral-<size>; random weights, one GPU, no RPC)")
+                         "--compare-family family beside the --compare-with family (default: Mixtral) at equal layer "
+                         "sizes, e.g. '2k,4k' (presets <family>-<size>; random weights, one GPU, no RPC)")
     ap.add_argument("--compare-family", default="sapapel",
-                    help="--compare-families: the family measured beside the Mixtral family (sapapel, kivezen)")
+                    help="--compare-families: the family measured beside the --compare-with family (sapapel, kivezen, "
+                         "nopunex)")
+    ap.add_argument("--compare-with", default="mixtral",
+                    help="--compare-families: the family measured beside it at equal layer sizes (mixtral; kivezen for nopunex)")
     ap.add_argument("--compare-batch", type=int, default=32, help="--compare-families: sequences")
     ap.add_argument("--compare-prompt", type=int, default=1024, help="--compare-families: prompt tokens per sequence")
     ap.add_argument("--compare-decode", type=int, default=128, help="--compare-families: decoded tokens per sequence")
@@ -488,7 +491,7 @@ def compare_families(args) -> int:
     rng = __import__("random").Random(args.seed)
     for item in [x for x in args.compare_families.split(",") if x]:
         size, _, only = item.partition(":")  # "2k" both families, "2k:sapapel" one (profiling)
-        for fam in ((only,) if only else (args.compare_family, "mixtral")):
+        for fam in ((only,) if only else (args.compare_family, args.compare_with)):
             name = f"{fam}-{size}"
             eng = LLMEngine(EngineConfig(model=name, seed=args.seed, max_num_seqs=B,
                                          max_num_batched_tokens=args.max_batched_tokens, max_model_len=max_len,

@@ -8,7 +8,7 @@
 //   latent_in         a projection row [query latent | key / value latent | shared key part]: both
 //                     latents set to unit RMS times a weight, the key part turned by the position;
 //                     the query latent is returned, [latent | key part] goes to the cache row
-//   latent_query      [folded query | the head's rotated part turned by the position] in fp32
+//   latent_query      [folded query | the head's rotated part turned by the position]
 //   masked_attention  query at position p sees keys lo(p) <= j <= p, lo(p) = max(0, p - window + 1,
 //                     floor(p / chunk) chunk); p_j = exp(s_j) / (exp(sink_h) + sum_j' exp(s_j')),
 //                     s = q . k * scale; o = sum_j p_j v_j.  Query head h reads key head h / (QH / KH)
@@ -104,16 +104,16 @@ latent_in_kernel(T* __restrict__ cq, T* __restrict__ cache, const T* __restrict_
 
 template <typename T>
 __global__ void __launch_bounds__(64)
-latent_query_kernel(float* __restrict__ out, const T* __restrict__ q_lat, const T* __restrict__ q,
+latent_query_kernel(T* __restrict__ out, const T* __restrict__ q_lat, const T* __restrict__ q,
                     const int* __restrict__ positions, const float* __restrict__ table, int pairs, int table_rows,
                     int halves, int T_, int H, int R, int D, int Dr) {
   const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
-  float* dst = out + (static_cast<int64_t>(t) * H + h) * (R + Dr);
+  T* dst = out + (static_cast<int64_t>(t) * H + h) * (R + Dr);
   const T* src = q_lat + (static_cast<int64_t>(h) * T_ + t) * R;
-  for (int i = lane; i < R; i += 64) dst[i] = ld<T>(src + i);
+  for (int i = lane; i < R; i += 64) dst[i] = src[i];
   if (Dr > 0) {
     const float* cs = table ? table + static_cast<int64_t>(clamp_pos(positions[t], table_rows)) * pairs * 2 : nullptr;
-    turn_head<T, float>(dst + R, q + (static_cast<int64_t>(t) * H + h) * (D + Dr) + D, Dr, cs, cs ? pairs : 0, halves, lane);
+    turn_head<T, T>(dst + R, q + (static_cast<int64_t>(t) * H + h) * (D + Dr) + D, Dr, cs, cs ? pairs : 0, halves, lane);
   }
 }
 
@@ -331,6 +331,225 @@ int launch_masked(const MaskedArgs& a, dim3 grid, hipStream_t stream) {
   return launch_one<T, 32, ALIAS>(a, grid, lds, stream);
 }
 
+// ---- bf16 on the matrix cores -------------------------------------------------------------------
+// NW waves of 16 (token, head) rows of one key head against 32-key tiles staged in LDS (pages hold
+// whole 32-key tiles; a tile is one contiguous run of the key cache).  Both products run transposed
+// on mfma_f32_16x16x32_bf16 so that the softmax weights never leave their registers:
+//
+//   S^T [keys x rows] = K [keys x D] . Q^T      A = key rows from LDS, B = the wave's Q (registers)
+//   O^T [V x rows]   += V^T [V x keys] . P^T    A = value columns from LDS, B = P^T from the S^T accumulators
+//
+// An accumulator lane (g4, n) holds query row n and keys 4 g4 .. 4 g4 + 3 of each 16-key half; the B
+// operand of the second product wants 8 key slots per lane, so slot (g4, e) is key 4 g4 + e of the
+// first half for e < 4 and key 16 + 4 g4 + e - 4 of the second.  The caches are key-major, so a
+// thread turns 4 keys x 8 value columns in registers and writes 8 column words of 4 keys into the
+// column-major LDS tile at those slots.  Scores are kept in log2 units.  Tiles of the next step are
+// fetched into registers before the current products.  A wave skips tiles outside its rows' bands.
+constexpr float kLog2e = 1.4426950408889634f;
+
+__host__ __device__ __forceinline__ int quad_slot(int q) { return (q & 3) * 8 + 4 * (q >> 2); }  // slot of key 4 q
+
+template <int D, int V, int NW, bool ALIAS>
+__global__ void __launch_bounds__(64 * NW) masked_attention_mfma_kernel(MaskedArgs a) {
+  constexpr int NT = 64 * NW, BQ = 16 * NW, BK = 32, NKK = D / 32, NRT = V / 16, CS = D + 8, CT = BK + 8;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  bf16_t* ks = reinterpret_cast<bf16_t*>(smem_raw);  // [BK][CS]  key-major
+  bf16_t* vt = ks + BK * CS;                          // [V][CT]   column-major, key slots permuted
+  const int QH = a.QH, KH = a.KH, bs = a.bs, R = QH / KH;
+  const int kh = blockIdx.y, vh = kh / (KH / a.VH);
+  int s = 0, tile = blockIdx.x;
+  for (; s < a.n_seqs; ++s) {
+    const int nt = ((a.cu_q[s + 1] - a.cu_q[s]) * R + BQ - 1) / BQ;
+    if (tile < nt) break;
+    tile -= nt;
+  }
+  if (s >= a.n_seqs) return;
+  const int q0 = a.cu_q[s], qlen = a.cu_q[s + 1] - q0, ctx = a.context_lens[s];
+  const int n_rows = qlen * R, row0 = tile * BQ;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, g = lane >> 4, n = lane & 15;
+  const int* bt = a.block_tables + static_cast<int64_t>(s) * a.bt_stride;
+  const int my_row = row0 + 16 * wave + n;
+  const bool valid = my_row < n_rows;
+  const int tl = valid ? my_row / R : 0, h = kh * R + (valid ? my_row - tl * R : 0);
+  const int my_pos = valid ? ctx - qlen + tl : -1;
+  const int my_lo = valid ? first_key(my_pos, a.window, a.chunk) : 0x7fffffff;
+  const int first_pos = ctx - qlen + row0 / R;
+  const int max_pos = ctx - qlen + (min(row0 + BQ, n_rows) - 1) / R;
+  const int k_begin = first_pos >= 0 ? first_key(first_pos, a.window, a.chunk) / BK * BK : 0;
+  const bf16_t* q = static_cast<const bf16_t*>(a.q);
+  const bf16_t* kc = static_cast<const bf16_t*>(a.k_cache);
+  const bf16_t* vc = static_cast<const bf16_t*>(a.v_cache);
+  const float sl2 = a.scale * kLog2e;
+
+  pk::bf16x8_t qf[NKK];
+  {
+    const bf16_t* qr = q + (static_cast<int64_t>(q0 + tl) * QH + h) * D + 8 * g;
+#pragma unroll
+    for (int kk = 0; kk < NKK; ++kk) {
+      pk::u32x4 v = {0u, 0u, 0u, 0u};
+      if (valid) v = *reinterpret_cast<const pk::u32x4*>(qr + kk * 32);
+      qf[kk] = __builtin_bit_cast(pk::bf16x8_t, v);
+    }
+  }
+  pk::f32x4 o[NRT];
+#pragma unroll
+  for (int rt = 0; rt < NRT; ++rt) o[rt] = pk::f32x4{0.f, 0.f, 0.f, 0.f};
+  float m_run = a.sink ? a.sink[h] * kLog2e : -INFINITY, l_run = a.sink ? 1.f : 0.f;
+
+  constexpr int KCH = BK * D / 8;          // 16-byte chunks of a key tile
+  constexpr int KIT = (KCH + NT - 1) / NT;
+  constexpr int VUN = V;                   // units of (4 keys x 8 value columns): 8 quads x V / 8 column chunks
+  constexpr int VIT = (VUN + NT - 1) / NT;
+  pk::u32x4 kv[KIT], vv[VIT][4];
+  auto fetch = [&](int k0) {
+    const int64_t blk = bt[k0 / bs];
+    const bf16_t* ksrc = kc + ((blk * KH + kh) * bs + k0 % bs) * D;
+    const bf16_t* vsrc = vc + ((blk * a.VH + vh) * bs + k0 % bs) * a.v_width;
+#pragma unroll
+    for (int i = 0; i < KIT; ++i) {
+      const int c = tid + NT * i;
+      if (c < KCH) kv[i] = *reinterpret_cast<const pk::u32x4*>(ksrc + c * 8);
+    }
+#pragma unroll
+    for (int i = 0; i < VIT; ++i) {
+      const int u = tid + NT * i;
+      if (u < VUN) {
+        const int qd = u & 7, c8 = u >> 3;
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          vv[i][j] = *reinterpret_cast<const pk::u32x4*>(vsrc + static_cast<int64_t>(4 * qd + j) * a.v_width + c8 * 8);
+      }
+    }
+  };
+  if (k_begin <= max_pos) fetch(k_begin);
+  for (int k0 = k_begin; k0 <= max_pos; k0 += BK) {
+#pragma unroll
+    for (int i = 0; i < KIT; ++i) {
+      const int c = tid + NT * i;
+      if (c < KCH) {
+        const int key = c / (D / 8), d8 = c - key * (D / 8);
+        *reinterpret_cast<pk::u32x4*>(ks + key * CS + d8 * 8) = kv[i];
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < VIT; ++i) {
+      const int u = tid + NT * i;
+      if (u < VUN) {
+        const int qd = u & 7, c8 = u >> 3;
+        bf16_t* dst = vt + (c8 * 8) * CT + quad_slot(qd);
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {  // columns 2 w (low halves) and 2 w + 1 (high halves) of the chunk
+          uint2 lo, hi;
+          lo.x = (vv[i][0][w] & 0xffffu) | (vv[i][1][w] << 16);
+          lo.y = (vv[i][2][w] & 0xffffu) | (vv[i][3][w] << 16);
+          hi.x = (vv[i][0][w] >> 16) | (vv[i][1][w] & 0xffff0000u);
+          hi.y = (vv[i][2][w] >> 16) | (vv[i][3][w] & 0xffff0000u);
+          *reinterpret_cast<uint2*>(dst + (2 * w) * CT) = lo;
+          *reinterpret_cast<uint2*>(dst + (2 * w + 1) * CT) = hi;
+        }
+      }
+    }
+    __syncthreads();
+    if (k0 + BK <= max_pos) fetch(k0 + BK);
+    if (__any(my_pos >= k0 && my_lo <= k0 + BK - 1)) {
+      pk::f32x4 sa[2] = {pk::f32x4{0.f, 0.f, 0.f, 0.f}, pk::f32x4{0.f, 0.f, 0.f, 0.f}};
+#pragma unroll
+      for (int sub = 0; sub < 2; ++sub) {
+        const bf16_t* kr = ks + (sub * 16 + n) * CS + 8 * g;
+#pragma unroll
+        for (int kk = 0; kk < NKK; ++kk)
+          sa[sub] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pk::ld8(kr + kk * 32), qf[kk], sa[sub], 0, 0, 0);
+      }
+      float sc[8];
+      float tmax = -INFINITY;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int key = k0 + (e >> 2) * 16 + 4 * g + (e & 3);
+        sc[e] = (key <= my_pos && key >= my_lo) ? sa[e >> 2][e & 3] * sl2 : -INFINITY;
+        tmax = fmaxf(tmax, sc[e]);
+      }
+      tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
+      tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+      const float m_new = fmaxf(m_run, tmax);
+      float p[8], tsum = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        p[e] = sc[e] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(sc[e] - m_new);
+        tsum += p[e];
+      }
+      tsum += __shfl_xor(tsum, 16, 64);
+      tsum += __shfl_xor(tsum, 32, 64);
+      const float resc = m_run == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m_run - m_new);
+      m_run = m_new;
+      l_run = l_run * resc + tsum;
+      pk::u32x4 pw;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) pw[e] = pk::pack2(p[2 * e], p[2 * e + 1]);
+      const pk::bf16x8_t pb = __builtin_bit_cast(pk::bf16x8_t, pw);
+      if (__any(resc != 1.f)) {
+#pragma unroll
+        for (int rt = 0; rt < NRT; ++rt) o[rt] *= resc;
+      }
+      const bf16_t* vr = vt + n * CT + 8 * g;
+#pragma unroll
+      for (int rt = 0; rt < NRT; ++rt)
+        o[rt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pk::ld8(vr + rt * 16 * CT), pb, o[rt], 0, 0, 0);
+    }
+    __syncthreads();
+  }
+  if (valid) {
+    const float inv = l_run > 0.f ? 1.f / l_run : 0.f;
+    const int64_t at = static_cast<int64_t>(q0 + tl) * a.out_ts + static_cast<int64_t>(h) * a.out_hs + 4 * g;
+#pragma unroll
+    for (int rt = 0; rt < NRT; ++rt) {
+      const float w0 = o[rt][0] * inv, w1 = o[rt][1] * inv, w2 = o[rt][2] * inv, w3 = o[rt][3] * inv;
+      if (a.out_f32) {
+        *reinterpret_cast<float4*>(static_cast<float*>(a.out) + at + rt * 16) = float4{w0, w1, w2, w3};
+      } else {
+        uint2 w;
+        w.x = pk::pack2(w0, w1);
+        w.y = pk::pack2(w2, w3);
+        *reinterpret_cast<uint2*>(static_cast<bf16_t*>(a.out) + at + rt * 16) = w;
+      }
+    }
+  }
+}
+
+template <int D, int V, int NW, bool ALIAS>
+int launch_mfma_one(const MaskedArgs& a, int T, hipStream_t stream) {
+  constexpr size_t lds = (32 * (D + 8) + V * 40) * sizeof(bf16_t);
+  auto kern = masked_attention_mfma_kernel<D, V, NW, ALIAS>;
+  if (lds > 60 * 1024) {
+    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                             static_cast<int>(lds));
+    if (e != hipSuccess) return static_cast<int>(e);
+  }
+  const int R = a.QH / a.KH;
+  const dim3 grid((T * R + 16 * NW - 1) / (16 * NW) + a.n_seqs, a.KH);
+  kern<<<grid, 64 * NW, lds, stream>>>(a);
+  return PK_CHECK_LAUNCH();
+}
+
+// head sizes the matrix-core kernel is built for; returns -100 when these are not among them
+int launch_mfma(const MaskedArgs& a, int T, bool alias, hipStream_t stream) {
+#define PKM_MM(DD, VV, NW, AL) \
+  if (a.D == DD && a.V == VV && alias == AL) return launch_mfma_one<DD, VV, NW, AL>(a, T, stream);
+  PKM_MM(64, 64, 8, false)
+  PKM_MM(64, 128, 8, false)
+  PKM_MM(128, 64, 8, false)
+  PKM_MM(128, 128, 8, false)
+  PKM_MM(96, 64, 8, true)
+  PKM_MM(160, 128, 8, true)
+  PKM_MM(192, 128, 8, true)
+  PKM_MM(288, 256, 4, true)
+  PKM_MM(320, 256, 4, true)
+  PKM_MM(576, 512, 4, true)
+#undef PKM_MM
+  return -100;
+}
+
+int g_masked_mfma = 1;  // 0: every launch takes the FMA kernel (tests compare the two)
+
 constexpr int kGateNone = 0, kGateSigmoid = 1, kGateSilu = 2;
 
 // one wave per (token, head)
@@ -401,7 +620,7 @@ PK_EXPORT int pkm_latent_in(void* cq, void* cache, const void* proj, long long s
   return PK_CHECK_LAUNCH();
 }
 
-// out [T, H, R + Dr] fp32; q_lat [H, T, R]; q [T, H, D + Dr]
+// out [T, H, R + Dr]; q_lat [H, T, R]; q [T, H, D + Dr], all of one element type
 PK_EXPORT int pkm_latent_query(void* out, const void* q_lat, const void* q, const void* positions, const void* table,
                                int pairs, int table_rows, int halves, int T, int H, int R, int D, int Dr, int dt,
                                hipStream_t stream) {
@@ -409,7 +628,7 @@ PK_EXPORT int pkm_latent_query(void* out, const void* q_lat, const void* q, cons
   if (2 * pairs > Dr || (table && table_rows < 1)) return -1;
   const dim3 grid(T, H);
   PKM_DISPATCH(dt, E, latent_query_kernel<E><<<grid, 64, 0, stream>>>(
-                          static_cast<float*>(out), static_cast<const E*>(q_lat), static_cast<const E*>(q),
+                          static_cast<E*>(out), static_cast<const E*>(q_lat), static_cast<const E*>(q),
                           static_cast<const int*>(positions), static_cast<const float*>(table), pairs, table_rows, halves,
                           T, H, R, D, Dr));
   return PK_CHECK_LAUNCH();
@@ -433,6 +652,10 @@ PK_EXPORT int pkm_masked_attention(void* out, long long out_ts, long long out_hs
                static_cast<const int*>(context_lens), static_cast<const float*>(sink), n_seqs, QH, KH, VH, D, V, bs, bk,
                scale, window, chunk};
   const int R = QH / KH;
+  if (g_masked_mfma && dt == kBF16 && q_dt == kBF16 && bs % 32 == 0 && v_width % 8 == 0) {
+    const int rc = launch_mfma(a, T, alias, stream);
+    if (rc != -100) return rc;
+  }
   // row tiles: every sequence adds at most one partly filled tile
   const int tiles = (T * R + kBQ - 1) / kBQ + n_seqs;
   const dim3 grid(tiles, KH);
@@ -440,6 +663,11 @@ PK_EXPORT int pkm_masked_attention(void* out, long long out_ts, long long out_hs
     PKM_DISPATCH(dt, E, return (launch_masked<E, true>(a, grid, stream)));
   }
   PKM_DISPATCH(dt, E, return (launch_masked<E, false>(a, grid, stream)));
+  return 0;
+}
+
+PK_EXPORT int pkm_set_masked_mfma(int on) {
+  g_masked_mfma = on;
   return 0;
 }
 

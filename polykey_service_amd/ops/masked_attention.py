@@ -170,14 +170,15 @@ def latent_in(proj: torch.Tensor, q_rank: int, R: int, Dr: int, wq: Optional[tor
 
 def latent_query(q_lat: torch.Tensor, q: torch.Tensor, D: int, Dr: int, positions: torch.Tensor,
                  table: Optional[torch.Tensor], halves: bool) -> torch.Tensor:
-    """q_lat [H, T, R] (queries folded into the latent space), q [T, H, D + Dr]: returns fp32
-    [T, H, R + Dr] = the folded query beside the head's rotated part turned by the position."""
+    """q_lat [H, T, R] (queries folded into the latent space), q [T, H, D + Dr]: returns
+    [T, H, R + Dr] = the folded query beside the head's rotated part turned by the position, in
+    the same element type."""
     H, T, R = q_lat.shape
-    out = torch.empty((T, H, R + Dr), dtype=torch.float32, device=q.device)
+    out = torch.empty((T, H, R + Dr), dtype=q.dtype, device=q.device)
     if not q.is_cuda:
-        out[..., :R] = q_lat.float().transpose(0, 1)
+        out[..., :R] = q_lat.transpose(0, 1)
         qr = q.float().view(T, H, D + Dr)[..., D:]
-        out[..., R:] = turn(qr, table[positions.long()], halves) if (table is not None and Dr) else qr
+        out[..., R:] = (turn(qr, table[positions.long()], halves) if (table is not None and Dr) else qr).to(q.dtype)
         return out
     assert q_lat.is_contiguous() and q.is_contiguous() and q.dtype == q_lat.dtype
     native.call("pkm_latent_query", out.data_ptr(), q_lat.data_ptr(), q.data_ptr(), positions.data_ptr(),

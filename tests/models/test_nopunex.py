@@ -279,6 +279,9 @@ def test_attention_sees_its_block_only(device, where, decoded):
         assert float(got[:12].min()) > 0.0
 
 
+MIX = {"attention": O.diff_attention, "latent_attention": O.latent_attention}
+
+
 def _latent_case(H, D, Dr, V, R, Q, window, W, scaling=(4.0, 64, 8.0, 1.0)):
     return O.make_config(pattern="m", heads=H, dim=D, rot_dim=Dr, vdim=V, kv_rank=R, q_rank=Q, window=window,
                          scaling=scaling)["layers"][0]["mixer"]
@@ -300,6 +303,46 @@ def test_latent_attention_mixer(device, H, D, Dr, V, R, Q, window):
     cache = (torch.zeros(8, 1, BS, R + Dr, device=dev),)
     got = _feed(mod, cache, h, [31, 2, 33, 1, 1, 7], [5, 0, 3], dev)
     close(got, want, 3e-4)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("kind,m", [
+    ("attention", dict(heads=8, kv_heads=2, dim=64, vdim=64, rot_dims=32, chunk=100)),
+    ("attention", dict(heads=4, kv_heads=4, dim=128, vdim=128, rot_dims=128, chunk=70)),
+    ("attention", dict(heads=6, kv_heads=1, dim=64, vdim=128, rot_dims=0, chunk=1000)),
+    ("latent_attention", dict(heads=16, dim=32, rot_dim=64, vdim=24, kv_rank=512, q_rank=40, window=90)),
+    ("latent_attention", dict(heads=5, dim=48, rot_dim=32, vdim=40, kv_rank=256, q_rank=64, window=33)),
+    ("latent_attention", dict(heads=3, dim=16, rot_dim=32, vdim=16, kv_rank=128, q_rank=32, window=400))])
+def test_matrix_core_attention(kind, m):
+    """bf16 at head sizes the MFMA kernel tiles: prompt portions that start and end inside 32-key
+    tiles, bands whose edges lie inside tiles, decoded tokens; against the plain rule and the FMA kernel."""
+    from polykey_service_amd.ops import native
+    dev, n, W = torch.device("cuda"), 330, 64
+    mm = O.make_config(pattern="a" if kind == "attention" else "m", **m)["layers"][0]["mixer"]
+    w = {k: v.bfloat16().double() for k, v in _weights(kind, mm, W, seed=m["heads"]).items()}
+    torch.manual_seed(1)
+    h = (torch.randn(n, W) * 0.5).bfloat16().float()
+    want = MIX[kind](h.double(), w, "", mm, 1e-5).float()
+    pages = [9, 3, 0, 7, 5, 1, 8, 2, 6, 4, 10]
+    portions = [150, 2, 37, 120] + [1] * 21
+
+    def run():
+        mod, spec = _mixer(kind, mm, w, W, dev, n, torch.bfloat16)
+        if kind == "attention":
+            cache = _attn_cache(spec, 12, dev, torch.bfloat16)
+        else:
+            cache = (torch.zeros(12, 1, BS, spec.kv_rank + spec.rot_dim, device=dev, dtype=torch.bfloat16),)
+        return _feed(mod, cache, h, portions, pages, dev, dtype=torch.bfloat16)
+    got = run()
+    native.call("pkm_set_masked_mfma", 0)
+    try:
+        fma = run()
+    finally:
+        native.call("pkm_set_masked_mfma", 1)
+    scale = float(want.pow(2).mean().sqrt())
+    assert float((fma - want).pow(2).mean(-1).sqrt().max()) < 0.05 * scale
+    assert float((got - want).pow(2).mean(-1).sqrt().max()) < 0.05 * scale
+    assert float((got - fma).pow(2).mean(-1).sqrt().max()) < 0.03 * scale
 
 
 @pytest.mark.parametrize("device", DEVICES)
