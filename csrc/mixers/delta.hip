@@ -9,7 +9,7 @@
 //                  S <- gate S ;  u = beta (v - S^T k) ;  S <- S + k u^T ;  o = S^T q
 //
 // The state of a (sequence, head) lives in the sequence's state slot between steps.  In delta_rule a
-// wave owns 16 value columns; the 4 lanes of a column hold key rows sub, sub + 4, ... of it in
+// wave owns 16 value columns; the 4 lanes of a column each hold a quarter of its key rows in
 // registers and sum their parts with two lane exchanges, in the same order for every token whether
 // it arrives in a long prompt portion or alone.  The first token of a portion reads the slot unless
 // it is position 0; the state after the portion's last token is written back.
@@ -93,19 +93,32 @@ conv_state_kernel(float* __restrict__ conv_state, const T* __restrict__ proj, in
 }
 
 constexpr int kMaxChunk = 16;  // tokens staged per group (fewer when a head is wide)
-constexpr int kCols = 64;   // value columns per workgroup (4 waves x 16)
+constexpr int kCols = 64;      // value columns per workgroup (4 waves x 16)
 
-// AT: element type of the a | b pre-activations.  ND = ceil(D / 4) key rows per lane.
+// sums over the 4 lanes of a quad (data-parallel lane exchanges inside the quad)
+__device__ __forceinline__ float quad_sum(float v) {
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xF, 0xF, false));
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xF, 0xF, false));
+  return v;
+}
+
+// AT: element type of the a | b pre-activations.  Lane `sub` of a column's quad keeps key rows
+// sub * nd .. sub * nd + nd - 1 (nd = ceil(D / 4) <= ND; rows past D hold zeros) in registers; q and
+// k of a token lie in LDS as 4 runs of ND (+ 4 floats of padding, so the quad's four 16-byte reads
+// fall on different banks).  The next group's q, k, v are fetched into registers before the
+// current group is computed.
 template <typename AT, int ND>
 __global__ void __launch_bounds__(256)
 delta_rule_kernel(float* __restrict__ out, const float* __restrict__ qkv, const AT* __restrict__ ab, int64_t ab_stride,
                   const float* __restrict__ a_log, const float* __restrict__ dt_bias, float* __restrict__ state,
                   const int* __restrict__ cu_q, const int* __restrict__ positions, const int* __restrict__ slots, int G, int D,
                   int H, int V, int kChunk) {
-  extern __shared__ float smem[];
-  float* qs = smem;                 // [kChunk][D]
-  float* ks = qs + kChunk * D;      // [kChunk][D]
-  float* vs = ks + kChunk * D;      // [kChunk][kCols]
+  constexpr int RS = ND + 4, TS = 4 * RS;          // floats per run and per token
+  constexpr int QK_IT = (kMaxChunk * 4 * ND + 255) / 256, V_IT = (kMaxChunk * kCols + 255) / 256;
+  extern __shared__ __attribute__((aligned(16))) float smem[];
+  float* qs = smem;                 // [kChunk][4][RS]
+  float* ks = qs + kChunk * TS;     // [kChunk][4][RS]
+  float* vs = ks + kChunk * TS;     // [kChunk][kCols]
   float* gs = vs + kChunk * kCols;  // [kChunk] gate
   float* bs_ = gs + kChunk;         // [kChunk] beta
   const int s = blockIdx.x / H, h = blockIdx.x - s * H;
@@ -115,6 +128,7 @@ delta_rule_kernel(float* __restrict__ out, const float* __restrict__ qkv, const 
   const int tid = threadIdx.x, sub = tid & 3, col = v0 + (tid >> 2);
   const int slot = slots[s];
   const int C = 2 * G * D + H * V;
+  const int nd = (D + 3) / 4;
   const int kvh = h / (H / G);
   const float neg_rate = -expf(a_log[h]), bias = dt_bias[h];
   float* sp = slot >= 0 ? state + ((static_cast<int64_t>(slot) * H + h) * D) * V : nullptr;
@@ -122,23 +136,46 @@ delta_rule_kernel(float* __restrict__ out, const float* __restrict__ qkv, const 
   float S[ND];
 #pragma unroll
   for (int i = 0; i < ND; ++i) {
-    const int d = sub + 4 * i;
-    S[i] = (carry && d < D && col < V) ? sp[static_cast<int64_t>(d) * V + col] : 0.f;
+    const int d = sub * nd + i;
+    S[i] = (carry && i < nd && d < D && col < V) ? sp[static_cast<int64_t>(d) * V + col] : 0.f;
   }
   const int64_t qo = static_cast<int64_t>(kvh) * D, ko = static_cast<int64_t>(G + kvh) * D;
   const int64_t vo = 2 * static_cast<int64_t>(G) * D + static_cast<int64_t>(h) * V + v0;
+  float rq[QK_IT], rk[QK_IT], rv[V_IT];
+  auto fetch = [&](int t0) {  // the group starting at token t0 (zeros outside the head's D rows)
+    const int nt = min(kChunk, b - t0);
+#pragma unroll
+    for (int i = 0; i < QK_IT; ++i) {
+      const int e = tid + 256 * i, t = e / (4 * ND), r = e - t * 4 * ND, su = r / ND, ii = r - su * ND;
+      const int d = su * nd + ii;
+      const bool ok = t < nt && ii < nd && d < D;
+      const float* row = qkv + static_cast<int64_t>(t0 + (ok ? t : 0)) * C;
+      rq[i] = ok ? row[qo + d] : 0.f;
+      rk[i] = ok ? row[ko + d] : 0.f;
+    }
+#pragma unroll
+    for (int i = 0; i < V_IT; ++i) {
+      const int e = tid + 256 * i, t = e / kCols, c = e - t * kCols;
+      const bool ok = t < nt && v0 + c < V;
+      rv[i] = ok ? qkv[static_cast<int64_t>(t0 + t) * C + vo + c] : 0.f;
+    }
+  };
+  fetch(a);
   for (int t0 = a; t0 < b; t0 += kChunk) {
     const int nt = min(kChunk, b - t0);
-    __syncthreads();
-    for (int e = tid; e < nt * D; e += 256) {
-      const int t = e / D, d = e - t * D;
-      const float* row = qkv + static_cast<int64_t>(t0 + t) * C;
-      qs[e] = row[qo + d];
-      ks[e] = row[ko + d];
+    __syncthreads();  // the group before has been read
+#pragma unroll
+    for (int i = 0; i < QK_IT; ++i) {
+      const int e = tid + 256 * i, t = e / (4 * ND), r = e - t * 4 * ND, su = r / ND, ii = r - su * ND;
+      if (t < kChunk) {
+        qs[t * TS + su * RS + ii] = rq[i];
+        ks[t * TS + su * RS + ii] = rk[i];
+      }
     }
-    for (int e = tid; e < nt * kCols; e += 256) {
-      const int t = e / kCols, c = e - t * kCols;
-      vs[e] = v0 + c < V ? qkv[static_cast<int64_t>(t0 + t) * C + vo + c] : 0.f;
+#pragma unroll
+    for (int i = 0; i < V_IT; ++i) {
+      const int e = tid + 256 * i;
+      if (e < kChunk * kCols) vs[e] = rv[i];
     }
     if (tid < nt) {
       const AT* r = ab + static_cast<int64_t>(t0 + tid) * ab_stride;
@@ -146,40 +183,45 @@ delta_rule_kernel(float* __restrict__ out, const float* __restrict__ qkv, const 
       bs_[tid] = sigmoidf(ld<AT>(r + H + h));
     }
     __syncthreads();
+    if (t0 + kChunk < b) fetch(t0 + kChunk);  // in flight while this group is computed
     for (int t = 0; t < nt; ++t) {
       const float gate = gs[t], beta = bs_[t];
       const float vv = vs[t * kCols + (tid >> 2)];
-      const float* kr = ks + t * D + sub;
-      const float* qr = qs + t * D + sub;
-      float r = 0.f;
+      const float4* kr = reinterpret_cast<const float4*>(ks + t * TS + sub * RS);
+      const float4* qr = reinterpret_cast<const float4*>(qs + t * TS + sub * RS);
+      float r0 = 0.f, r1 = 0.f, r2 = 0.f, r3 = 0.f;
 #pragma unroll
-      for (int i = 0; i < ND; ++i) {
-        if (sub + 4 * i < D) {
-          S[i] *= gate;
-          r += S[i] * kr[4 * i];
-        }
+      for (int i = 0; i < ND / 4; ++i) {
+        const float4 k4 = kr[i];
+        r0 += S[4 * i] * k4.x;
+        r1 += S[4 * i + 1] * k4.y;
+        r2 += S[4 * i + 2] * k4.z;
+        r3 += S[4 * i + 3] * k4.w;
       }
-      r += __shfl_xor(r, 1, 64);
-      r += __shfl_xor(r, 2, 64);
+      const float r = gate * quad_sum((r0 + r1) + (r2 + r3));  // (gate S)^T k
       const float u = beta * (vv - r);
-      float o = 0.f;
+      float o0 = 0.f, o1 = 0.f, o2 = 0.f, o3 = 0.f;
 #pragma unroll
-      for (int i = 0; i < ND; ++i) {
-        if (sub + 4 * i < D) {
-          S[i] += kr[4 * i] * u;
-          o += S[i] * qr[4 * i];
-        }
+      for (int i = 0; i < ND / 4; ++i) {
+        const float4 k4 = kr[i], q4 = qr[i];
+        S[4 * i] = gate * S[4 * i] + k4.x * u;
+        o0 += S[4 * i] * q4.x;
+        S[4 * i + 1] = gate * S[4 * i + 1] + k4.y * u;
+        o1 += S[4 * i + 1] * q4.y;
+        S[4 * i + 2] = gate * S[4 * i + 2] + k4.z * u;
+        o2 += S[4 * i + 2] * q4.z;
+        S[4 * i + 3] = gate * S[4 * i + 3] + k4.w * u;
+        o3 += S[4 * i + 3] * q4.w;
       }
-      o += __shfl_xor(o, 1, 64);
-      o += __shfl_xor(o, 2, 64);
+      const float o = quad_sum((o0 + o1) + (o2 + o3));
       if (sub == 0 && col < V) out[(static_cast<int64_t>(t0 + t) * H + h) * V + col] = o;
     }
   }
   if (sp != nullptr && col < V) {
 #pragma unroll
     for (int i = 0; i < ND; ++i) {
-      const int d = sub + 4 * i;
-      if (d < D) sp[static_cast<int64_t>(d) * V + col] = S[i];
+      const int d = sub * nd + i;
+      if (i < nd && d < D) sp[static_cast<int64_t>(d) * V + col] = S[i];
     }
   }
 }
@@ -218,9 +260,11 @@ PK_EXPORT int pkm_delta_rule(void* out, const void* qkv, const void* ab, long lo
   if (n_seqs <= 0 || T <= 0) return 0;
   if (D < 1 || D > 512 || V < 1 || G < 1 || H % G) return -1;
   const dim3 grid(n_seqs * H, (V + kCols - 1) / kCols);
-  const int chunk = max(1, min(kMaxChunk, 15360 / (2 * D + kCols + 2)));  // at most 60 KiB of LDS
-  const size_t lds = (static_cast<size_t>(chunk) * (2 * D + kCols) + 2 * chunk) * sizeof(float);
   const int nd = (D + 3) / 4;
+  const int ndt = nd <= 8 ? 8 : nd <= 16 ? 16 : nd <= 32 ? 32 : nd <= 64 ? 64 : 128;
+  const int per_tok = 8 * (ndt + 4) + kCols + 2;  // floats of LDS per staged token
+  const int chunk = max(1, min(kMaxChunk, 15360 / per_tok));  // at most 60 KiB of LDS
+  const size_t lds = static_cast<size_t>(chunk) * per_tok * sizeof(float);
 #define PKM_DELTA(ND)                                                                                                 \
   PKM_DISPATCH(ab_dt, E, delta_rule_kernel<E, ND><<<grid, 256, lds, stream>>>(                                          \
                              static_cast<float*>(out), static_cast<const float*>(qkv), static_cast<const E*>(ab), ab_stride, \

@@ -46,6 +46,15 @@ from .kivezen import _p, _packed, _project
 from .weights import SafetensorsIndex, random_full
 
 
+def _pad_rows(w: torch.Tensor) -> torch.Tensor:
+    """Zero rows up to a multiple of 128 where the decode GEMM could then tile the projection (its
+    input width a multiple of 256); the extra output columns are never read."""
+    n, k = w.shape
+    if k % 256 or n % 128 == 0:
+        return w
+    return torch.cat([w, w.new_zeros((128 - n % 128, k))], 0)
+
+
 class DiffAttention(nn.Module):
     """Weights of one differential-attention mixer.  Query rows are stored per key / value group as
     (first maps of the group's heads, second maps of the group's heads): query "head" i of 2H then
@@ -71,7 +80,7 @@ class DiffAttention(nn.Module):
         assert s.rot is None or (s.rot.dims % 2 == 0 and s.rot.dims <= D)
         r = H // G
         q = q.reshape(G, r, 2, D, W).permute(0, 2, 1, 3, 4).reshape(2 * H * D, W)
-        self.w_in = _p(torch.cat([q, k, v, g], 0).to(device=device, dtype=dtype))
+        self.w_in = _p(_pad_rows(torch.cat([q, k, v, g], 0)).to(device=device, dtype=dtype))
         self.w_o = _p(o.to(device=device, dtype=dtype))
         dot = lambda a, b: float((a.double().reshape(-1) * b.double().reshape(-1)).sum())
         self.lam = math.exp(dot(lq1, lk1)) - math.exp(dot(lq2, lk2)) + s.diff
@@ -85,7 +94,7 @@ class DiffAttention(nn.Module):
                                 2 * H, 2 * G, G, D, V)
         a = ma_ops.masked_attention(q, cache[0], cache[1], V, md.block_tables, md.cu_q, md.context_lens, md.num_seqs,
                                     s.scale, chunk=s.chunk)
-        o = ma_ops.head_norm_gate(a, H, V, eps, proj[:, n:], ma_ops.GATE_SIGMOID, h.dtype, post=1.0 - s.diff,
+        o = ma_ops.head_norm_gate(a, H, V, eps, proj[:, n:n + H * V], ma_ops.GATE_SIGMOID, h.dtype, post=1.0 - s.diff,
                                   pair_group=H // G, coef=self.lam)
         return _project(o, self.w_o, self.w_o_p, partial=True)
 
@@ -118,7 +127,7 @@ class WindowLatentAttention(nn.Module):
         assert s.rot is None or (s.rot.dims % 2 == 0 and s.rot.dims <= Dr)
         to = lambda t: _p(t.to(device=device, dtype=dtype))
         f32 = lambda t: _p(t.to(device=device, dtype=torch.float32).reshape(-1))
-        self.w_in, self.uq, self.w_o = to(torch.cat([dq, dkv], 0)), to(uq), to(o)
+        self.w_in, self.uq, self.w_o = to(_pad_rows(torch.cat([dq, dkv], 0))), to(uq), to(o)
         self.uk = to(uk.reshape(H, D, R))
         self.uv_t = to(uv.reshape(H, V, R).transpose(1, 2))
         self.q_norm, self.kv_norm, self.sink = f32(dq_norm), f32(dkv_norm), f32(sink)
@@ -129,7 +138,7 @@ class WindowLatentAttention(nn.Module):
         H, D, Dr, V, R = s.heads, s.dim, s.rot_dim, s.vdim, s.kv_rank
         T = h.shape[0]
         proj = _project(h, self.w_in, self.w_in_p)
-        cq = ma_ops.latent_in(proj, s.q_rank, R, Dr, self.q_norm, self.kv_norm, eps, positions, md.slot_mapping,
+        cq = ma_ops.latent_in(proj[:, :s.q_rank + R + Dr], s.q_rank, R, Dr, self.q_norm, self.kv_norm, eps, positions, md.slot_mapping,
                               self.table, True, cache[0])
         q = _project(cq, self.uq, self.uq_p)
         q_lat = torch.bmm(q.view(T, H, D + Dr)[:, :, :D].transpose(0, 1), self.uk)                  # [H, T, R]
@@ -163,7 +172,7 @@ class DeltaMixer(nn.Module):
         assert q.shape == (G * D, W) == k.shape and v.shape == (H * V, W) == g.shape and o.shape == (W, H * V)
         assert a.shape == (H, W) == b.shape and qc.shape == (G * D, K) == kc.shape and vc.shape == (H * V, K)
         f32 = lambda t: _p(t.to(device=device, dtype=torch.float32).reshape(-1))
-        self.w_in = _p(torch.cat([q, k, v, a, b, g], 0).to(device=device, dtype=dtype))
+        self.w_in = _p(_pad_rows(torch.cat([q, k, v, a, b, g], 0)).to(device=device, dtype=dtype))
         self.w_o = _p(o.to(device=device, dtype=dtype))
         self.taps = _p(torch.cat([qc, kc, vc], 0).to(device=device, dtype=torch.float32))
         self.a_log, self.dt_bias, self.norm_w = f32(a_log), f32(dt_bias), f32(norm_w)
@@ -178,7 +187,7 @@ class DeltaMixer(nn.Module):
                                   md.token_seq, G, D, H, V)
         o = delta_ops.delta_rule(qkv, proj[:, C:C + 2 * H], self.a_log, self.dt_bias, cache[0], md.cu_q, md.num_seqs,
                                  positions, md.state_slots, G, D, H, V)
-        z = ma_ops.head_norm_gate(o, H, V, eps, proj[:, C + 2 * H:], ma_ops.GATE_SILU, h.dtype, weight=self.norm_w)
+        z = ma_ops.head_norm_gate(o, H, V, eps, proj[:, C + 2 * H:C + 2 * H + H * V], ma_ops.GATE_SILU, h.dtype, weight=self.norm_w)
         return _project(z, self.w_o, self.w_o_p, partial=True)
 
 
