@@ -142,9 +142,115 @@ __global__ void __launch_bounds__(kThreads) sandwich_kernel(SandwichArgs a) {
   }
 }
 
+template <typename E>
+__device__ __forceinline__ float4 ld4(const E* p);
+template <>
+__device__ __forceinline__ float4 ld4<float>(const float* p) { return *reinterpret_cast<const float4*>(p); }
+template <>
+__device__ __forceinline__ float4 ld4<bf16_t>(const bf16_t* p) {
+  const uint2 w = *reinterpret_cast<const uint2*>(p);
+  return float4{__uint_as_float(w.x << 16), __uint_as_float(w.x & 0xffff0000u), __uint_as_float(w.y << 16),
+                __uint_as_float(w.y & 0xffff0000u)};
+}
+template <typename E>
+__device__ __forceinline__ void st4(E* p, float4 v);
+template <>
+__device__ __forceinline__ void st4<float>(float* p, float4 v) { *reinterpret_cast<float4*>(p) = v; }
+template <>
+__device__ __forceinline__ void st4<bf16_t>(bf16_t* p, float4 v) {
+  uint2 w;
+  w.x = pk::pack2(v.x, v.y);
+  w.y = pk::pack2(v.z, v.w);
+  *reinterpret_cast<uint2*>(p) = w;
+}
+
+// The same step for W % 4 == 0, W <= 4 * kVecGroups * kThreads: four consecutive coordinates per
+// thread and group, 16-byte accesses of the fp32 rows, the row stays in registers between passes.
+constexpr int kVecGroups = 4;
+
+template <typename YT, typename AT>
+__global__ void __launch_bounds__(kThreads) sandwich_vec_kernel(SandwichArgs a) {
+  __shared__ float red[16];
+  const int r = blockIdx.x, tid = threadIdx.x, W = a.W;
+  const int t = a.rows ? a.rows[r] : r;
+  float* xr = a.x + static_cast<int64_t>(t) * W;
+  float4 v[kVecGroups];
+  auto stats = [&](float& mean, float& rstd) {
+    float s = 0.f;
+#pragma unroll
+    for (int g = 0; g < kVecGroups; ++g) s += (v[g].x + v[g].y) + (v[g].z + v[g].w);
+    mean = pk::block_sum(s, red) / static_cast<float>(W);
+    float q = 0.f;
+#pragma unroll
+    for (int g = 0; g < kVecGroups; ++g) {
+      if (4 * (tid + g * kThreads) < W) {
+        const float d0 = v[g].x - mean, d1 = v[g].y - mean, d2 = v[g].z - mean, d3 = v[g].w - mean;
+        q += (d0 * d0 + d1 * d1) + (d2 * d2 + d3 * d3);
+      }
+    }
+    rstd = 1.f / sqrtf(pk::block_sum(q, red) / static_cast<float>(W) + a.eps);
+  };
+  auto norm4 = [](float4 z, float mean, float rstd, float4 w, float4 b) {
+    return float4{(z.x - mean) * rstd * w.x + b.x, (z.y - mean) * rstd * w.y + b.y, (z.z - mean) * rstd * w.z + b.z,
+                  (z.w - mean) * rstd * w.w + b.w};
+  };
+  float mean = 0.f, rstd = 1.f;
+  if (a.y) {
+    const YT* yr = static_cast<const YT*>(a.y) + static_cast<int64_t>(t) * W;
+#pragma unroll
+    for (int g = 0; g < kVecGroups; ++g) {
+      const int c = 4 * (tid + g * kThreads);
+      v[g] = float4{0.f, 0.f, 0.f, 0.f};
+      if (c < W) {
+        v[g] = ld4<YT>(yr + c);
+        for (int s = 1; s < a.nslab; ++s) {
+          const float4 z = ld4<YT>(yr + s * a.slab_stride + c);
+          v[g].x += z.x, v[g].y += z.y, v[g].z += z.z, v[g].w += z.w;
+        }
+      }
+    }
+    if (a.pw) stats(mean, rstd);
+#pragma unroll
+    for (int g = 0; g < kVecGroups; ++g) {
+      const int c = 4 * (tid + g * kThreads);
+      if (c < W) {
+        float4 z = v[g];
+        if (a.pw) z = norm4(z, mean, rstd, ld4<float>(a.pw + c), ld4<float>(a.pb + c));
+        if (a.replace) {
+          if (a.add) {
+            const float4 d = ld4<float>(a.add + c);
+            z.x += d.x, z.y += d.y, z.z += d.z, z.w += d.w;
+          }
+        } else {
+          const float4 x = ld4<float>(xr + c);
+          z.x += x.x, z.y += x.y, z.z += x.z, z.w += x.w;
+        }
+        st4<float>(xr + c, z);
+        v[g] = z;
+      }
+    }
+  } else {
+#pragma unroll
+    for (int g = 0; g < kVecGroups; ++g) {
+      const int c = 4 * (tid + g * kThreads);
+      v[g] = c < W ? ld4<float>(xr + c) : float4{0.f, 0.f, 0.f, 0.f};
+    }
+  }
+  if (!a.ow) return;
+  stats(mean, rstd);
+  AT* out = static_cast<AT*>(a.act) + static_cast<int64_t>(r) * W;
+#pragma unroll
+  for (int g = 0; g < kVecGroups; ++g) {
+    const int c = 4 * (tid + g * kThreads);
+    if (c < W) st4<AT>(out + c, norm4(v[g], mean, rstd, ld4<float>(a.ow + c), ld4<float>(a.ob + c)));
+  }
+}
+
 template <typename YT, typename AT>
 int launch_sandwich(const SandwichArgs& a, int R, hipStream_t stream) {
-  if (a.W <= kMaxPer * kThreads) {
+  if (a.W % 4 == 0 && a.W <= 4 * kVecGroups * kThreads) {
+    sandwich_vec_kernel<YT, AT><<<R, kThreads, 0, stream>>>(a);
+  } else if (a.W <= kMaxPer * kThreads) {
     sandwich_kernel<YT, AT, true><<<R, kThreads, 0, stream>>>(a);
   } else {
     sandwich_kernel<YT, AT, false><<<R, kThreads, static_cast<size_t>(a.W) * sizeof(float), stream>>>(a);
@@ -176,6 +282,23 @@ __global__ void __launch_bounds__(256) silu_mul_kernel(T* __restrict__ out, cons
     u += ld<IN>(row + s * slab_stride + F + c);
   }
   st<T>(out + t * F + c, g / (1.f + expf(-g)) * u);
+}
+
+template <typename IN, typename T>
+__global__ void __launch_bounds__(256) silu_mul_vec_kernel(T* __restrict__ out, const IN* __restrict__ gu, int F, int nslab,
+                                                           int64_t slab_stride) {
+  const int64_t t = blockIdx.y;
+  const int c = 4 * (blockIdx.x * blockDim.x + threadIdx.x);
+  if (c >= F) return;
+  const IN* row = gu + t * 2 * F;
+  float4 g = ld4<IN>(row + c), u = ld4<IN>(row + F + c);
+  for (int s = 1; s < nslab; ++s) {
+    const float4 g2 = ld4<IN>(row + s * slab_stride + c), u2 = ld4<IN>(row + s * slab_stride + F + c);
+    g.x += g2.x, g.y += g2.y, g.z += g2.z, g.w += g2.w;
+    u.x += u2.x, u.y += u2.y, u.z += u2.z, u.w += u2.w;
+  }
+  auto f = [](float gg, float uu) { return gg / (1.f + expf(-gg)) * uu; };
+  st4<T>(out + t * F + c, float4{f(g.x, u.x), f(g.y, u.y), f(g.z, u.z), f(g.w, u.w)});
 }
 
 __global__ void __launch_bounds__(256) scale_kernel(float* __restrict__ x, int64_t n, float k) {
@@ -218,8 +341,21 @@ PK_EXPORT int pkm_join_cast(void* out, const void* x, const void* x0, int T, int
 PK_EXPORT int pkm_silu_mul(void* out, const void* gu, int T, int F, int nslab, int in_dt, int out_dt, hipStream_t stream) {
   if (T <= 0 || F <= 0) return 0;
   if (nslab < 1 || (nslab > 1 && in_dt != kF32)) return -1;
-  const dim3 grid((F + 255) / 256, T);
   const int64_t ss = static_cast<int64_t>(T) * 2 * F;
+  if (F % 4 == 0) {
+    const dim3 vgrid((F / 4 + 255) / 256, T);
+    if (in_dt == kF32) {
+      PKM_DISPATCH(out_dt, E, silu_mul_vec_kernel<float, E><<<vgrid, 256, 0, stream>>>(
+                                  static_cast<E*>(out), static_cast<const float*>(gu), F, nslab, ss));
+    } else if (in_dt == kBF16) {
+      PKM_DISPATCH(out_dt, E, silu_mul_vec_kernel<bf16_t, E><<<vgrid, 256, 0, stream>>>(
+                                  static_cast<E*>(out), static_cast<const bf16_t*>(gu), F, 1, ss));
+    } else {
+      return -2;
+    }
+    return PK_CHECK_LAUNCH();
+  }
+  const dim3 grid((F + 255) / 256, T);
   if (in_dt == kF32) {
     PKM_DISPATCH(out_dt, E, silu_mul_kernel<float, E><<<grid, 256, 0, stream>>>(static_cast<E*>(out),
                                                                                  static_cast<const float*>(gu), F, nslab, ss));
