@@ -137,6 +137,11 @@ struct MaskedArgs {
   int n_seqs, QH, KH, VH, D, V, bs, BK;
   float scale;
   int window, chunk;
+  // decoded tokens on the matrix cores: the band's keys cut into n_parts runs of `part` keys,
+  // partial sums in the workspace (merged by masked_merge_kernel)
+  int part, n_parts;
+  float* ws_o;   // [n_seqs, n_parts, QH, V] unnormalised
+  float* ws_ml;  // [n_seqs, n_parts, QH, 2] (max in log2 units, sum)
 };
 
 __device__ __forceinline__ int first_key(int pos, int window, int chunk) {
@@ -349,7 +354,9 @@ constexpr float kLog2e = 1.4426950408889634f;
 
 __host__ __device__ __forceinline__ int quad_slot(int q) { return (q & 3) * 8 + 4 * (q >> 2); }  // slot of key 4 q
 
-template <int D, int V, int NW, bool ALIAS>
+// SPLIT: one token per sequence; blockIdx.z picks a run of a.part keys of the band and the
+// workgroup leaves (max, sum, unnormalised o) per row in the workspace (no sink: the merge adds it).
+template <int D, int V, int NW, bool ALIAS, bool SPLIT>
 __global__ void __launch_bounds__(64 * NW) masked_attention_mfma_kernel(MaskedArgs a) {
   constexpr int NT = 64 * NW, BQ = 16 * NW, BK = 32, NKK = D / 32, NRT = V / 16, CS = D + 8, CT = BK + 8;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
@@ -358,12 +365,18 @@ __global__ void __launch_bounds__(64 * NW) masked_attention_mfma_kernel(MaskedAr
   const int QH = a.QH, KH = a.KH, bs = a.bs, R = QH / KH;
   const int kh = blockIdx.y, vh = kh / (KH / a.VH);
   int s = 0, tile = blockIdx.x;
-  for (; s < a.n_seqs; ++s) {
-    const int nt = ((a.cu_q[s + 1] - a.cu_q[s]) * R + BQ - 1) / BQ;
-    if (tile < nt) break;
-    tile -= nt;
+  if (SPLIT) {
+    const int ntile = (R + BQ - 1) / BQ;
+    s = blockIdx.x / ntile;
+    tile = blockIdx.x - s * ntile;
+  } else {
+    for (; s < a.n_seqs; ++s) {
+      const int nt = ((a.cu_q[s + 1] - a.cu_q[s]) * R + BQ - 1) / BQ;
+      if (tile < nt) break;
+      tile -= nt;
+    }
+    if (s >= a.n_seqs) return;
   }
-  if (s >= a.n_seqs) return;
   const int q0 = a.cu_q[s], qlen = a.cu_q[s + 1] - q0, ctx = a.context_lens[s];
   const int n_rows = qlen * R, row0 = tile * BQ;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, g = lane >> 4, n = lane & 15;
@@ -374,8 +387,12 @@ __global__ void __launch_bounds__(64 * NW) masked_attention_mfma_kernel(MaskedAr
   const int my_pos = valid ? ctx - qlen + tl : -1;
   const int my_lo = valid ? first_key(my_pos, a.window, a.chunk) : 0x7fffffff;
   const int first_pos = ctx - qlen + row0 / R;
-  const int max_pos = ctx - qlen + (min(row0 + BQ, n_rows) - 1) / R;
-  const int k_begin = first_pos >= 0 ? first_key(first_pos, a.window, a.chunk) / BK * BK : 0;
+  int max_pos = ctx - qlen + (min(row0 + BQ, n_rows) - 1) / R;
+  int k_begin = first_pos >= 0 ? first_key(first_pos, a.window, a.chunk) / BK * BK : 0;
+  if (SPLIT) {
+    k_begin += blockIdx.z * a.part;
+    max_pos = min(max_pos, k_begin + a.part - 1);
+  }
   const bf16_t* q = static_cast<const bf16_t*>(a.q);
   const bf16_t* kc = static_cast<const bf16_t*>(a.k_cache);
   const bf16_t* vc = static_cast<const bf16_t*>(a.v_cache);
@@ -394,7 +411,8 @@ __global__ void __launch_bounds__(64 * NW) masked_attention_mfma_kernel(MaskedAr
   pk::f32x4 o[NRT];
 #pragma unroll
   for (int rt = 0; rt < NRT; ++rt) o[rt] = pk::f32x4{0.f, 0.f, 0.f, 0.f};
-  float m_run = a.sink ? a.sink[h] * kLog2e : -INFINITY, l_run = a.sink ? 1.f : 0.f;
+  const bool with_sink = !SPLIT && a.sink != nullptr;
+  float m_run = with_sink ? a.sink[h] * kLog2e : -INFINITY, l_run = with_sink ? 1.f : 0.f;
 
   constexpr int KCH = BK * D / 8;          // 16-byte chunks of a key tile
   constexpr int KIT = (KCH + NT - 1) / NT;
@@ -497,6 +515,19 @@ __global__ void __launch_bounds__(64 * NW) masked_attention_mfma_kernel(MaskedAr
     }
     __syncthreads();
   }
+  if (SPLIT) {
+    if (valid) {
+      const int64_t at = (static_cast<int64_t>(s) * a.n_parts + blockIdx.z) * QH + h;
+#pragma unroll
+      for (int rt = 0; rt < NRT; ++rt)
+        *reinterpret_cast<float4*>(a.ws_o + at * V + rt * 16 + 4 * g) = float4{o[rt][0], o[rt][1], o[rt][2], o[rt][3]};
+      if (g == 0) {
+        a.ws_ml[at * 2] = m_run;
+        a.ws_ml[at * 2 + 1] = l_run;
+      }
+    }
+    return;
+  }
   if (valid) {
     const float inv = l_run > 0.f ? 1.f / l_run : 0.f;
     const int64_t at = static_cast<int64_t>(q0 + tl) * a.out_ts + static_cast<int64_t>(h) * a.out_hs + 4 * g;
@@ -515,25 +546,70 @@ __global__ void __launch_bounds__(64 * NW) masked_attention_mfma_kernel(MaskedAr
   }
 }
 
-template <int D, int V, int NW, bool ALIAS>
+// out[token of sequence s, head h] from the runs' (max, sum, o) and the head's sink: one workgroup
+// per (sequence, head); the first wave turns the (at most 64) runs into one weight per run.
+template <typename T>
+__global__ void __launch_bounds__(128)
+masked_merge_kernel(void* __restrict__ out, int64_t out_ts, int64_t out_hs, int out_f32, const float* __restrict__ ws_o,
+                    const float* __restrict__ ws_ml, const int* __restrict__ cu_q, const float* __restrict__ sink,
+                    int n_parts, int QH, int V) {
+  __shared__ float wgt[64];
+  const int s = blockIdx.x, h = blockIdx.y;
+  const int tok = cu_q[s];
+  if (threadIdx.x < 64) {
+    const int p = threadIdx.x;
+    const int64_t at = (static_cast<int64_t>(s) * n_parts + p) * QH + h;
+    const float m = p < n_parts ? ws_ml[at * 2] : -INFINITY;
+    const float l = p < n_parts ? ws_ml[at * 2 + 1] : 0.f;
+    const float sk = sink ? sink[h] * kLog2e : -INFINITY;
+    const float M = pk::wave_max(fmaxf(m, sk));
+    const float w = m == -INFINITY ? 0.f : exp2f(m - M);
+    float L = pk::wave_sum(w * l);
+    if (sink) L += exp2f(sk - M);
+    wgt[p] = L > 0.f ? w / L : 0.f;
+  }
+  __syncthreads();
+  const int64_t at = static_cast<int64_t>(tok) * out_ts + static_cast<int64_t>(h) * out_hs;
+  const float* base = ws_o + (static_cast<int64_t>(s) * n_parts * QH + h) * V;
+  for (int c = threadIdx.x; c < V; c += blockDim.x) {
+    float u = 0.f;
+    for (int p = 0; p < n_parts; ++p) u += wgt[p] * base[static_cast<int64_t>(p) * QH * V + c];
+    if (out_f32) {
+      static_cast<float*>(out)[at + c] = u;
+    } else {
+      st<T>(static_cast<T*>(out) + at + c, u);
+    }
+  }
+}
+
+template <int D, int V, int NW, bool ALIAS, bool SPLIT>
 int launch_mfma_one(const MaskedArgs& a, int T, hipStream_t stream) {
   constexpr size_t lds = (32 * (D + 8) + V * 40) * sizeof(bf16_t);
-  auto kern = masked_attention_mfma_kernel<D, V, NW, ALIAS>;
+  auto kern = masked_attention_mfma_kernel<D, V, NW, ALIAS, SPLIT>;
   if (lds > 60 * 1024) {
     const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                              static_cast<int>(lds));
     if (e != hipSuccess) return static_cast<int>(e);
   }
   const int R = a.QH / a.KH;
-  const dim3 grid((T * R + 16 * NW - 1) / (16 * NW) + a.n_seqs, a.KH);
+  const dim3 grid = SPLIT ? dim3(a.n_seqs * ((R + 16 * NW - 1) / (16 * NW)), a.KH, a.n_parts)
+                          : dim3((T * R + 16 * NW - 1) / (16 * NW) + a.n_seqs, a.KH);
   kern<<<grid, 64 * NW, lds, stream>>>(a);
   return PK_CHECK_LAUNCH();
 }
 
-// head sizes the matrix-core kernel is built for; returns -100 when these are not among them
+// head sizes the matrix-core kernel is built for
+bool mfma_sizes(int D, int V, bool alias) {
+  if (!alias) return (D == 64 || D == 128) && (V == 64 || V == 128);
+  return (D == 96 && V == 64) || (D == 160 && V == 128) || (D == 192 && V == 128) || (D == 288 && V == 256) ||
+         (D == 320 && V == 256) || (D == 576 && V == 512);
+}
+
+// returns -100 when the sizes are not among those the matrix-core kernel is built for
+template <bool SPLIT>
 int launch_mfma(const MaskedArgs& a, int T, bool alias, hipStream_t stream) {
 #define PKM_MM(DD, VV, NW, AL) \
-  if (a.D == DD && a.V == VV && alias == AL) return launch_mfma_one<DD, VV, NW, AL>(a, T, stream);
+  if (a.D == DD && a.V == VV && alias == AL) return launch_mfma_one<DD, VV, NW, AL, SPLIT>(a, T, stream);
   PKM_MM(64, 64, 8, false)
   PKM_MM(64, 128, 8, false)
   PKM_MM(128, 64, 8, false)
@@ -639,7 +715,8 @@ PK_EXPORT int pkm_masked_attention(void* out, long long out_ts, long long out_hs
                                    const void* k_cache, const void* v_cache, int v_width, const void* block_tables,
                                    long long bt_stride, const void* cu_q, const void* context_lens, const void* sink,
                                    int n_seqs, int T, int QH, int KH, int VH, int D, int V, int bs, float scale, int window,
-                                   int chunk, int dt, hipStream_t stream) {
+                                   int chunk, int num_decode, void* ws_o, void* ws_ml, int part, int n_parts, int dt,
+                                   hipStream_t stream) {
   if (n_seqs <= 0 || T <= 0) return 0;
   if (KH < 1 || VH < 1 || QH % KH || KH % VH || V < 1 || V > 512 || V > v_width || D < 1) return -1;
   if ((q_dt != dt && q_dt != kF32) || (out_dt != dt && out_dt != kF32)) return -1;
@@ -650,11 +727,36 @@ PK_EXPORT int pkm_masked_attention(void* out, long long out_ts, long long out_hs
   MaskedArgs a{out, out_ts, out_hs, out_dt == kF32, q, q_dt == kF32, k_cache, v_cache, v_width,
                static_cast<const int*>(block_tables), bt_stride, static_cast<const int*>(cu_q),
                static_cast<const int*>(context_lens), static_cast<const float*>(sink), n_seqs, QH, KH, VH, D, V, bs, bk,
-               scale, window, chunk};
+               scale, window, chunk, 0, 1, nullptr, nullptr};
   const int R = QH / KH;
-  if (g_masked_mfma && dt == kBF16 && q_dt == kBF16 && bs % 32 == 0 && v_width % 8 == 0) {
-    const int rc = launch_mfma(a, T, alias, stream);
-    if (rc != -100) return rc;
+  if (g_masked_mfma && dt == kBF16 && q_dt == kBF16 && bs % 32 == 0 && v_width % 8 == 0 && mfma_sizes(D, V, alias)) {
+    // the first num_decode sequences hold one token each: their bands are cut into runs when a
+    // workspace is given (ws_o [num_decode, n_parts, QH, V], ws_ml [num_decode, n_parts, QH, 2] fp32)
+    const int nd = (ws_o && ws_ml && n_parts > 1) ? (num_decode < n_seqs ? num_decode : n_seqs) : 0;
+    if (nd > 0) {
+      if (part < 32 || part % 32 || n_parts > 64) return -1;
+      MaskedArgs d = a;
+      d.n_seqs = nd;
+      d.part = part;
+      d.n_parts = n_parts;
+      d.ws_o = static_cast<float*>(ws_o);
+      d.ws_ml = static_cast<float*>(ws_ml);
+      int rc = launch_mfma<true>(d, nd, alias, stream);
+      if (rc) return rc;
+      masked_merge_kernel<bf16_t><<<dim3(nd, QH), 128, 0, stream>>>(out, out_ts, out_hs, a.out_f32, d.ws_o, d.ws_ml, d.cu_q,
+                                                                    d.sink, n_parts, QH, V);
+      rc = PK_CHECK_LAUNCH();
+      if (rc) return rc;
+    }
+    if (n_seqs > nd) {
+      MaskedArgs p = a;
+      p.n_seqs = n_seqs - nd;
+      p.block_tables += static_cast<int64_t>(nd) * bt_stride;
+      p.cu_q += nd;
+      p.context_lens += nd;
+      return launch_mfma<false>(p, T - nd, alias, stream);
+    }
+    return 0;
   }
   // row tiles: every sequence adds at most one partly filled tile
   const int tiles = (T * R + kBQ - 1) / kBQ + n_seqs;
@@ -664,6 +766,24 @@ PK_EXPORT int pkm_masked_attention(void* out, long long out_ts, long long out_hs
   }
   PKM_DISPATCH(dt, E, return (launch_masked<E, false>(a, grid, stream)));
   return 0;
+}
+
+// Keys per run of a decoded token's band (a multiple of 32), 0: no split.  `capacity`: the most
+// cached tokens of a sequence; the band spans at most window + 31 / chunk + 31 keys from its
+// aligned start.  Runs are at least 64 keys, at most 64 of them, and aim at ~512 workgroups per launch.
+PK_EXPORT int pkm_masked_decode_part(int nd, int QH, int KH, int D, int V, int alias, int bs, int capacity, int window,
+                                     int chunk, int dt) {
+  if (!g_masked_mfma || dt != kBF16 || bs % 32 || nd <= 0 || !mfma_sizes(D, V, alias != 0)) return 0;
+  int span = capacity;
+  if (window > 0 && window + 31 < span) span = window + 31;
+  if (chunk > 0 && chunk + 31 < span) span = chunk + 31;
+  span = (span + 31) / 32 * 32;
+  const int wgs = nd * KH;
+  int want = (512 + wgs - 1) / wgs;  // runs wanted
+  if (want > 64) want = 64;
+  if (want > span / 64) want = span / 64;
+  if (want <= 1) return 0;
+  return ((span + want - 1) / want + 31) / 32 * 32;
 }
 
 PK_EXPORT int pkm_set_masked_mfma(int on) {

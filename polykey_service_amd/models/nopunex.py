@@ -93,7 +93,7 @@ class DiffAttention(nn.Module):
         q = ma_ops.rotate_cache(proj[:, :n], positions, md.slot_mapping, self.table, True, cache[0], cache[1],
                                 2 * H, 2 * G, G, D, V)
         a = ma_ops.masked_attention(q, cache[0], cache[1], V, md.block_tables, md.cu_q, md.context_lens, md.num_seqs,
-                                    s.scale, chunk=s.chunk)
+                                    s.scale, chunk=s.chunk, num_decode=md.num_decode)
         o = ma_ops.head_norm_gate(a, H, V, eps, proj[:, n:n + H * V], ma_ops.GATE_SIGMOID, h.dtype, post=1.0 - s.diff,
                                   pair_group=H // G, coef=self.lam)
         return _project(o, self.w_o, self.w_o_p, partial=True)
@@ -145,7 +145,7 @@ class WindowLatentAttention(nn.Module):
         qf = ma_ops.latent_query(q_lat, q, D, Dr, positions, self.table, True)
         o_lat = ma_ops.masked_attention(qf, cache[0], None, R, md.block_tables, md.cu_q, md.context_lens, md.num_seqs,
                                         s.scale, window=s.window, sink=self.sink if s.sink else None,
-                                        out_dtype=h.dtype, head_major=True)                        # [H, T, R]
+                                        out_dtype=h.dtype, head_major=True, num_decode=md.num_decode)                        # [H, T, R]
         o = torch.bmm(o_lat, self.uv_t).transpose(0, 1).reshape(T, H * V)
         return _project(o, self.w_o, self.w_o_p, partial=True)
 

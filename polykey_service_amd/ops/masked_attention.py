@@ -87,12 +87,13 @@ def rotate_cache(proj: torch.Tensor, positions: torch.Tensor, slot_mapping: torc
 def masked_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: Optional[torch.Tensor], V: int,
                      block_tables: torch.Tensor, cu_q: torch.Tensor, context_lens: torch.Tensor, n_seqs: int,
                      scale: float, window: int = 0, chunk: int = 0, sink: Optional[torch.Tensor] = None,
-                     out_dtype: torch.dtype = torch.float32, head_major: bool = False) -> torch.Tensor:
+                     out_dtype: torch.dtype = torch.float32, head_major: bool = False, num_decode: int = 0) -> torch.Tensor:
     """q [T, QH, D] (fp32 or the cache's dtype); sequence s owns tokens cu_q[s]:cu_q[s+1], the LAST
     ones of its context_lens[s] cached tokens.  ``v_cache`` None: the value of a key is the first
     ``V`` numbers of its key row (key heads = value heads).  ``sink`` [QH] fp32 logits or None.
-    Returns [T, QH, V], or [QH, T, V] with ``head_major``, in ``out_dtype``.  Scores, softmax and the
-    value sums are fp32."""
+    The first ``num_decode`` sequences hold one token each (the matrix-core kernel cuts their bands
+    into runs that a second kernel merges).  Returns [T, QH, V], or [QH, T, V] with ``head_major``,
+    in ``out_dtype``.  Scores, softmax and the value sums are fp32."""
     T, QH, D = q.shape
     KH, bs = k_cache.shape[1], k_cache.shape[2]
     vc = k_cache if v_cache is None else v_cache
@@ -131,10 +132,28 @@ def masked_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: Optional[t
     assert block_tables.stride(1) == 1 and (sink is None or (sink.dtype == torch.float32 and sink.numel() == QH))
     assert q.dtype in (torch.float32, k_cache.dtype)
     ts, hs = (V, T * V) if head_major else (QH * V, V)
+    nd = min(num_decode, n_seqs)
+    ws_o = ws_ml = None
+    part = n_parts = 0
+    if nd and q.dtype == k_cache.dtype:
+        capacity = block_tables.shape[1] * bs
+        part = native.mixers().pkm_masked_decode_part(nd, QH, KH, D, V, int(v_cache is None), bs, capacity, int(window),
+                                                      int(chunk), native.dt_code(k_cache.dtype))
+        if part > 0:
+            span = capacity
+            if window > 0:
+                span = min(span, window + 31)
+            if chunk > 0:
+                span = min(span, chunk + 31)
+            n_parts = -(-((span + 31) // 32 * 32) // part)
+            if n_parts > 1:
+                ws_o = torch.empty((nd, n_parts, QH, V), dtype=torch.float32, device=q.device)
+                ws_ml = torch.empty((nd, n_parts, QH, 2), dtype=torch.float32, device=q.device)
     native.call("pkm_masked_attention", out.data_ptr(), ts, hs, native.dt_code(out_dtype), q.data_ptr(),
                 native.dt_code(q.dtype), k_cache.data_ptr(), vc.data_ptr(), vc.shape[3], block_tables.data_ptr(),
                 block_tables.stride(0), cu_q.data_ptr(), context_lens.data_ptr(), native.ptr(sink), n_seqs, T, QH, KH, VH,
-                D, V, bs, float(scale), int(window), int(chunk), native.dt_code(k_cache.dtype), native.stream_ptr())
+                D, V, bs, float(scale), int(window), int(chunk), nd, native.ptr(ws_o), native.ptr(ws_ml), part, n_parts,
+                native.dt_code(k_cache.dtype), native.stream_ptr())
     return out
 
 

@@ -108,7 +108,8 @@ MIXER_SIGNATURES = {
     "pkm_latent_in": [P, P, P, I64, I32, I32, I32, P, P, F32, P, P, P, I32, I32, I32, I32, I32, I32, P],
     "pkm_latent_query": [P, P, P, P, P, I32, I32, I32, I32, I32, I32, I32, I32, I32, P],
     "pkm_masked_attention": [P, I64, I64, I32, P, I32, P, P, I32, P, I64, P, P, P, I32, I32, I32, I32, I32, I32, I32, I32,
-                             F32, I32, I32, I32, P],
+                             F32, I32, I32, I32, P, P, I32, I32, I32, P],
+    "pkm_masked_decode_part": [I32, I32, I32, I32, I32, I32, I32, I32, I32, I32, I32],
     "pkm_set_masked_mfma": [I32],
     "pkm_head_norm_gate": [P, P, I32, I32, I32, F32, P, I64, I32, I32, P, F32, I32, F32, I32, P],
     "pkm_conv_unit": [P, P, I64, P, I32, P, P, P, P, P, I32, I32, I32, I32, I32, I32, I32, P],

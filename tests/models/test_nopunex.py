@@ -593,3 +593,33 @@ def test_bfloat16_stays_near_the_plain_model(small):
     rel = lambda a, b: (a - b).pow(2).mean(-1).sqrt() / b.pow(2).mean(-1).sqrt()
     assert float(rel(got, want).mean()) < 0.1 and float(rel(got, want).median()) < 0.08
     assert float(rel(got, ref).mean()) < 0.03
+
+
+@pytest.mark.gpu
+def test_matrix_core_sizes_in_mixed_batches(tmp_path):
+    """A bf16 model at sizes the matrix-core attention kernel tiles: unequal live requests, prompt
+    portions beside decoded tokens (whose bands are cut into runs and merged), decode graphs;
+    against the ops' compositions at the same precision and the plain model."""
+    cfg = O.make_config(vocab=120, width=128, pattern="AMDA", heads=4, kv_heads=2, dim=64, vdim=64, rot_dims=32, ff=128,
+                        chunk=100, window=150, kv_rank=128, q_rank=64, rot_dim=32, conv=4, loop=(1, 3, 2))
+    w = O.random_model(cfg, seed=12, std=0.12)
+    path = checkpoint(tmp_path, cfg, w)
+    lens = {"a": 300, "b": 170, "c": 230, "d": 40}
+    toks = {k: rand_tokens(n, cfg["vocab"], 30 + i) for i, (k, n) in enumerate(lens.items())}
+    plans = {"a": cut("a", toks["a"], [200, 60]), "b": cut("b", toks["b"], [2, 150]), "c": cut("c", toks["c"], [64, 64, 90]),
+             "d": cut("d", toks["d"], [33])}
+    steps, live = [], list(lens)
+    while live:
+        step = []
+        for rid in list(live):
+            step.append(plans[rid].pop(0))
+            if not plans[rid]:
+                live.remove(rid)
+        steps.append(step)
+    got = replay(engine(path, "cuda", dtype="bfloat16", pool_tokens=1024, budget=1024, graphs=True), steps)
+    ref = replay(engine(path, "cpu", dtype="bfloat16", pool_tokens=1024, budget=1024), steps)
+    rel = lambda a, b: (a - b).pow(2).mean(-1).sqrt() / b.pow(2).mean(-1).sqrt()
+    for rid, n in lens.items():
+        g, r = rows_of(got, rid, n), rows_of(ref, rid, n)
+        assert float(rel(g, r).mean()) < 0.03, rid
+        assert float(rel(g, O.forward(cfg, w, toks[rid]).float()).median()) < 0.1, rid
