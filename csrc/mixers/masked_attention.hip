@@ -350,6 +350,7 @@ int launch_masked(const MaskedArgs& a, dim3 grid, hipStream_t stream) {
 // thread turns 4 keys x 8 value columns in registers and writes 8 column words of 4 keys into the
 // column-major LDS tile at those slots.  Scores are kept in log2 units.  Tiles of the next step are
 // fetched into registers before the current products.  A wave skips tiles outside its rows' bands.
+// Row tiles are dealt to the XCDs in contiguous ranges, so tiles that share keys share an L2.
 constexpr float kLog2e = 1.4426950408889634f;
 
 __host__ __device__ __forceinline__ int quad_slot(int q) { return (q & 3) * 8 + 4 * (q >> 2); }  // slot of key 4 q
@@ -370,6 +371,9 @@ __global__ void __launch_bounds__(64 * NW) masked_attention_mfma_kernel(MaskedAr
     s = blockIdx.x / ntile;
     tile = blockIdx.x - s * ntile;
   } else {
+    // workgroups go to the 8 XCDs round-robin: XCD x takes the x-th eighth of the row tiles (gridDim.x
+    // is a multiple of 8), so neighbouring tiles, which share most of their keys, share one L2
+    tile = (blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);
     for (; s < a.n_seqs; ++s) {
       const int nt = ((a.cu_q[s + 1] - a.cu_q[s]) * R + BQ - 1) / BQ;
       if (tile < nt) break;
@@ -593,7 +597,7 @@ int launch_mfma_one(const MaskedArgs& a, int T, hipStream_t stream) {
   }
   const int R = a.QH / a.KH;
   const dim3 grid = SPLIT ? dim3(a.n_seqs * ((R + 16 * NW - 1) / (16 * NW)), a.KH, a.n_parts)
-                          : dim3((T * R + 16 * NW - 1) / (16 * NW) + a.n_seqs, a.KH);
+                          : dim3(((T * R + 16 * NW - 1) / (16 * NW) + a.n_seqs + 7) / 8 * 8, a.KH);
   kern<<<grid, 64 * NW, lds, stream>>>(a);
   return PK_CHECK_LAUNCH();
 }
