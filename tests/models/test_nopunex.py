@@ -310,6 +310,10 @@ def test_latent_attention_mixer(device, H, D, Dr, V, R, Q, window):
     ("attention", dict(heads=8, kv_heads=2, dim=64, vdim=64, rot_dims=32, chunk=100)),
     ("attention", dict(heads=4, kv_heads=4, dim=128, vdim=128, rot_dims=128, chunk=70)),
     ("attention", dict(heads=6, kv_heads=1, dim=64, vdim=128, rot_dims=0, chunk=1000)),
+    ("attention", dict(heads=2, kv_heads=1, dim=128, vdim=64, rot_dims=64, chunk=32)),
+    ("latent_attention", dict(heads=4, dim=24, rot_dim=32, vdim=24, kv_rank=64, q_rank=40, window=96)),
+    ("latent_attention", dict(heads=20, dim=32, rot_dim=64, vdim=16, kv_rank=128, q_rank=32, window=64)),
+    ("latent_attention", dict(heads=2, dim=64, rot_dim=64, vdim=64, kv_rank=256, q_rank=48, window=1)),
     ("latent_attention", dict(heads=16, dim=32, rot_dim=64, vdim=24, kv_rank=512, q_rank=40, window=90)),
     ("latent_attention", dict(heads=5, dim=48, rot_dim=32, vdim=40, kv_rank=256, q_rank=64, window=33)),
     ("latent_attention", dict(heads=3, dim=16, rot_dim=32, vdim=16, kv_rank=128, q_rank=32, window=400))])
