@@ -555,7 +555,7 @@ PRESETS["kivezen-4k"] = KivezenConfig.uniform("kivezen-4k", 32000, 4096, "LAAA",
 
 
 PRESETS["tiny-nopunex"] = NopunexConfig.uniform("tiny-nopunex", 512, 128, "AdMA", 4, 2, 32, 256, kv_rank=48, q_rank=64,
-                                                rot_dim=16, window=40, chunk=24, loop=(1, 3, 2))
+                                                rot_dim=8, window=40, chunk=24, loop=(1, 3, 2))
 # speed measurements beside kivezen-2k / kivezen-4k (the closest family: fp32 stream, a recurrent
 # mixer among attention layers): the same width, depth, heads, KV heads and head size, dense
 # feed-forwards of the MoE's active size
