@@ -563,6 +563,52 @@ def test_other_sizes_and_loop_positions(device, tmp_path, kw):
     close(rows_of(got, "a", 80), O.forward(cfg, w, toks), 5e-4)
 
 
+def _drawn_config(seed):
+    """A configuration drawn from the seed: layer order, loop, head counts and every size."""
+    r = random.Random(seed)
+    kv = r.choice([1, 2, 3, 4])
+    heads = kv * r.choice([1, 2, 3, 4])
+    nl = r.randint(3, 6)
+    pattern = "".join(r.choice("AMD") if r.random() < 0.75 else r.choice("amd") for _ in range(nl))
+    a = r.randint(0, nl - 1)
+    loop = (a, r.randint(a + 1, nl), r.randint(1, 3)) if r.random() < 0.8 else None
+    dim = r.choice([16, 24, 40, 64, 80])
+    return O.make_config(vocab=r.randint(100, 300), width=r.choice([64, 96, 160]), pattern=pattern, heads=heads, kv_heads=kv,
+                         dim=dim, vdim=r.choice([16, 24, 48, 72, 128]), rot_dims=r.choice([0, 2, dim // 4 * 2, dim]),
+                         ff=r.choice([64, 100, 200]), chunk=r.choice([16, 30, 100]), window=r.choice([8, 31, 100]),
+                         kv_rank=r.choice([32, 48, 80, 128]), q_rank=r.choice([32, 72, 136]), rot_dim=r.choice([8, 24, 32, 64]),
+                         conv=r.randint(2, 5), loop=loop, diff=r.choice([0.2, 0.35]),
+                         scaling=r.choice([None, (4.0, 64, 8.0, 1.0)]), logit_scale=r.choice([1.0, 2.0, 0.5]))
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("seed", [1, 2, 3, 4, 5, 6])
+def test_drawn_configurations_in_mixed_steps(device, tmp_path, seed):
+    """Layer orders, loops and sizes drawn at random, three unequal requests in steps drawn at
+    random (a request may sit out a step), against the plain model."""
+    cfg = _drawn_config(seed)
+    w = O.random_model(cfg, seed=seed, std=0.1)
+    r = random.Random(100 + seed)
+    lens = {"a": r.randint(100, 200), "b": r.randint(2, 60), "c": r.randint(40, 150)}
+    toks = {k: rand_tokens(n, cfg["vocab"], seed * 7 + i) for i, (k, n) in enumerate(lens.items())}
+    plans = {k: cut(k, toks[k], [r.choice([2, 3, 17, 33, 64]) for _ in range(r.randint(1, 5))]) for k in lens}
+    steps, live = [], list(lens)
+    while live:
+        step = []
+        for rid in list(live):
+            if r.random() < 0.85 or len(live) == 1:
+                step.append(plans[rid].pop(0))
+                if not plans[rid]:
+                    live.remove(rid)
+        if step:
+            steps.append(step)
+    got = replay(engine(checkpoint(tmp_path, cfg, w), device), steps)
+    for rid, n in lens.items():
+        want = O.forward(cfg, w, toks[rid])
+        err = (rows_of(got, rid, n).double() - want).pow(2).mean(-1).sqrt() / want.pow(2).mean(-1).sqrt()
+        assert float(err.max()) < 1e-3, (rid, cfg["layers"])
+
+
 @pytest.mark.parametrize("device", DEVICES)
 def test_greedy_generation_through_the_engine(device, small):
     """add_request / step with the scheduler's own batching: two prompts generated together equal
