@@ -612,18 +612,20 @@ bool mfma_sizes(int D, int V, bool alias) {
 // returns -100 when the sizes are not among those the matrix-core kernel is built for
 template <bool SPLIT>
 int launch_mfma(const MaskedArgs& a, int T, bool alias, hipStream_t stream) {
-#define PKM_MM(DD, VV, NW, AL) \
-  if (a.D == DD && a.V == VV && alias == AL) return launch_mfma_one<DD, VV, NW, AL, SPLIT>(a, T, stream);
-  PKM_MM(64, 64, 8, false)
-  PKM_MM(64, 128, 8, false)
-  PKM_MM(128, 64, 8, false)
-  PKM_MM(128, 128, 8, false)
-  PKM_MM(96, 64, 8, true)
-  PKM_MM(160, 128, 8, true)
-  PKM_MM(192, 128, 8, true)
-  PKM_MM(288, 256, 4, true)
-  PKM_MM(320, 256, 4, true)
-  PKM_MM(576, 512, 4, true)
+#define PKM_MM(DD, VV, NW, NWS, AL) \
+  if (a.D == DD && a.V == VV && alias == AL) return launch_mfma_one<DD, VV, (SPLIT ? NWS : NW), AL, SPLIT>(a, T, stream);
+  // waves per workgroup for prompt portions / for decoded tokens (one 16-row tile computes there:
+  // fewer, less loaded waves stage the tiles faster for the wide rows)
+  PKM_MM(64, 64, 8, 8, false)
+  PKM_MM(64, 128, 8, 8, false)
+  PKM_MM(128, 64, 8, 8, false)
+  PKM_MM(128, 128, 8, 8, false)
+  PKM_MM(96, 64, 8, 8, true)
+  PKM_MM(160, 128, 8, 8, true)
+  PKM_MM(192, 128, 8, 8, true)
+  PKM_MM(288, 256, 8, 4, true)
+  PKM_MM(320, 256, 8, 4, true)
+  PKM_MM(576, 512, 8, 4, true)
 #undef PKM_MM
   return -100;
 }
