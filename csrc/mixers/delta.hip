@@ -22,7 +22,7 @@ namespace {
 __device__ __forceinline__ float siluf(float z) { return z / (1.f + expf(-z)); }
 __device__ __forceinline__ float softplusf(float z) { return fmaxf(z, 0.f) + log1pf(expf(-fabsf(z))); }
 
-constexpr int kMaxTaps = 8;
+constexpr int kMaxTaps = 64;  // the kernels loop over the taps; this only bounds a wrong argument
 
 // one wave per (token, head): heads 0..G-1 q, G..2G-1 k, then H value heads
 template <typename T>
