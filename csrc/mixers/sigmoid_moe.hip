@@ -96,7 +96,8 @@ __device__ __forceinline__ bool find_tile(const int* offsets, int E, int tile, i
 
 // C[r, n] = sum_k A[arow(r), k] * B[e][n, k]   (B: [E, N, K]); DUAL: a second B and a gated
 // epilogue: with slot_scale the scaled SiLU product, without it the clamped product
-// min(g, limit) * sigmoid(1.702 min(g, limit)) * (clamp(u, -limit, limit) + 1).  256 threads: thread (ty, tx) owns rows ty, ty + 16 and columns tx, tx + 16.
+// min(g, limit) * sigmoid(1.702 min(g, limit)) * (clamp(u, -limit, limit) + 1), or with limit <= 0 the plain
+// SiLU product silu(g) * u.  256 threads: thread (ty, tx) owns rows ty, ty + 16 and columns tx, tx + 16.
 template <typename T, typename TA, typename TC, bool DUAL>
 __global__ void __launch_bounds__(256)
 grouped_rows_kernel(TC* __restrict__ C, const TA* __restrict__ A, const T* __restrict__ B0, const T* __restrict__ B1,
@@ -160,9 +161,11 @@ grouped_rows_kernel(TC* __restrict__ C, const TA* __restrict__ A, const T* __res
       if (DUAL && slot_scale) {
         const float g = s * v, u = s * acc1[i][j];
         v = g * sigmoidf(g) * u;
-      } else if (DUAL) {
+      } else if (DUAL && limit > 0.f) {
         const float g = fminf(v, limit), u = fminf(fmaxf(acc1[i][j], -limit), limit);
         v = g * sigmoidf(1.702f * g) * (u + 1.f);
+      } else if (DUAL) {
+        v = v * sigmoidf(v) * acc1[i][j];
       }
       st<TC>(C + static_cast<int64_t>(r) * N + n, v);
     }
@@ -257,7 +260,8 @@ PK_EXPORT int pkm_expert_gate_up(void* h, const void* x, const void* gate, const
   return PK_CHECK_LAUNCH();
 }
 
-// the same with the clamped epilogue (no scores): h = min(g, limit) sigmoid(1.702 min(g, limit)) (clamp(u) + 1)
+// the same with the clamped epilogue (no scores): h = min(g, limit) sigmoid(1.702 min(g, limit)) (clamp(u) + 1);
+// limit <= 0: h = silu(g) u
 PK_EXPORT int pkm_expert_gate_up_clamped(void* h, const void* x, const void* gate, const void* up, const void* offsets,
                                          const void* sorted_slots, float limit, int n_rows, int top, int E, int F,
                                          int W, int dt, hipStream_t stream) {

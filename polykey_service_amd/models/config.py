@@ -532,9 +532,209 @@ class NopunexConfig:
                    loop=loop or (0, 0, 1), looped=loop is not None, logit_scale=1.0)
 
 
+@dataclasses.dataclass(frozen=True)
+class PooledWindowAttentionSpec:
+    """Grouped-query softmax attention whose projections (with biases) pass a causal per-channel
+    filter of ``conv`` taps (0 / 1: none), then a weighted unit RMS per head on q and k (``qk_norm``)
+    and a rotation.  A query sees the last ``window`` single keys (0: all) and, behind the window,
+    the mean key / value of every complete block of ``pool`` positions (0: none) that ended before
+    the window; scores are capped by tanh (``softcap`` 0: none); the denominator holds one learned
+    sink term per head (``sink``); the heads' softmax weights are mixed by an [H, H] matrix (``talk``)
+    before they meet the values of each head's own key / value head."""
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    scale: float
+    softcap: float = 0.0
+    rot: Optional[RotarySpec] = None
+    window: int = 0
+    pool: int = 0
+    conv: int = 0
+    qk_norm: bool = True
+    sink: bool = True
+    talk: bool = True
+    bias: bool = True
+
+
+@dataclasses.dataclass(frozen=True)
+class WkvSpec:
+    """Time mixing with a [dim, dim] fp32 state per head that decays per key channel by a
+    data-dependent factor exp(-exp(.)) from a low-rank projection (``decay_rank``), a bonus for the
+    current token, inputs mixed with the previous token's, unit RMS per head and a SiLU gate."""
+    heads: int
+    dim: int
+    decay_rank: int = 0     # read from the checkpoint's tensor shapes when 0
+
+
+@dataclasses.dataclass(frozen=True)
+class SelectiveScanSpec:
+    """State-space mixer with input-dependent step sizes: ``inner`` channels, each with a diagonal
+    state of ``state`` numbers, a causal filter of ``conv`` taps and SiLU in front, a gate behind."""
+    inner: int
+    state: int
+    dt_rank: int
+    conv: int
+
+
+@dataclasses.dataclass(frozen=True)
+class ParallelSpec:
+    """Two mixers reading the same input, their outputs summed with fixed weights."""
+    left: PooledWindowAttentionSpec
+    right: WkvSpec
+    left_scale: float = 1.0
+    right_scale: float = 1.0
+
+
+@dataclasses.dataclass(frozen=True)
+class ClampedFFSpec:
+    """down(min(g, limit) sigmoid(1.702 min(g, limit)) (clamp(u, -limit, limit) + 1)), g = gate x, u = up x."""
+    ff: int
+    limit: float
+
+
+@dataclasses.dataclass(frozen=True)
+class SoftmaxMoESpec:
+    """SiLU-gated experts chosen by the largest fp32 router logits, weighted by the softmax over the
+    chosen logits, plus an ungated shared expert of ``shared_ff`` (0: none)."""
+    experts: int
+    top: int
+    ff: int
+    shared_ff: int = 0
+
+
+@dataclasses.dataclass(frozen=True)
+class BibezenConfig:
+    """Bibezen: pre-norm layers (norm weights stored around zero) on ``streams`` fp32 residual
+    streams (hyper-connections; 0: the one plain residual) with sublayer outputs scaled by
+    ``residual_mult``; the mixer's input passes h + filter(h) over ``canon_taps`` positions (0: not);
+    mixers are ``wkv``, ``mamba1`` (selective scan) or ``parallel`` (pooled-window attention beside
+    wkv); feed-forwards are a clamped GLU, a softmax-routed mixture with a shared expert, or none.
+    The embedding rows are scaled by ``embed_scale``; the logits reuse the embedding table.  Read
+    from a checkpoint folder's config.json ("architecture": "Bibezen")."""
+    name: str
+    vocab_size: int
+    hidden_size: int
+    layers: tuple
+    rms_eps: float
+    streams: int = 0
+    residual_mult: float = 1.0
+    embed_scale: float = 1.0
+    canon_taps: int = 0
+    max_position: int = 1 << 20
+    bos_token_id: int = 0
+    eos_token_id: int = -1
+    init_std: float = 0.05
+    family: str = "bibezen"
+    is_moe: bool = False
+    experts_per_token: int = 0
+
+    @property
+    def num_layers(self) -> int:
+        return len(self.layers)
+
+    @property
+    def runs(self) -> tuple:
+        return tuple(range(len(self.layers)))
+
+    @property
+    def needs_state(self) -> bool:
+        return True     # every mixer keeps per-sequence state (filters, previous rows, recurrences)
+
+    def num_params(self) -> int:
+        W, n = self.hidden_size, self.vocab_size * self.hidden_size
+        wkv = lambda m: W * m.heads * m.dim * 5 + 2 * max(m.decay_rank, 1) * (W + m.heads * m.dim) // 2
+        att = lambda m: W * (2 * m.heads * m.dim + m.kv_heads * (m.dim + m.vdim)) + W * m.heads * (m.vdim - m.dim)
+        for l in self.layers:
+            m = l.mixer
+            if l.type == "wkv":
+                n += wkv(m)
+            elif l.type == "mamba1":
+                n += 3 * W * m.inner + m.inner * (m.dt_rank * 2 + 2 * m.state) + m.inner * m.state
+            else:
+                n += wkv(m.right) + att(m.left)
+            f = l.mlp
+            if isinstance(f, ClampedFFSpec):
+                n += 3 * W * f.ff
+            elif f is not None:
+                n += f.experts * (3 * f.ff * W + W) + 3 * f.shared_ff * W
+        return n
+
+    def kv_bytes_per_token(self, dtype_bytes: int = 2) -> int:
+        """Paged bytes per token: keys and values of every attention branch and the pages of their block means."""
+        return sum(2 * l.mixer.left.kv_heads * (l.mixer.left.dim + l.mixer.left.vdim) for l in self.layers
+                   if l.type == "parallel") * dtype_bytes
+
+    @staticmethod
+    def _left(m: dict) -> PooledWindowAttentionSpec:
+        r, mask = m.get("rot"), m.get("mask") or {}
+        rot = RotarySpec(int(r["dims"]), float(r["base"]), None, halves=True) if r else None
+        s = PooledWindowAttentionSpec(int(m["heads"]), int(m.get("kv_heads", m["heads"])), int(m["dim"]),
+                                      int(m.get("vdim", m["dim"])), float(m["scale"]), float(m.get("softcap") or 0.0), rot,
+                                      int(mask.get("size") or 0), int(mask.get("pool") or 0), int(m.get("conv") or 0))
+        if s.heads % s.kv_heads or (rot is not None and (rot.dims % 2 or rot.dims > s.dim)):
+            raise ValueError("Bibezen: heads must be a multiple of kv_heads and rot.dims even and at most dim")
+        return s
+
+    @classmethod
+    def from_json(cls, c: dict, name: str = "bibezen") -> "BibezenConfig":
+        layers = []
+        for l in c["layers"]:
+            m = l["mixer"]
+            if l["type"] == "wkv":
+                mixer = WkvSpec(int(m["heads"]), int(m["dim"]))
+            elif l["type"] == "mamba1":
+                mixer = SelectiveScanSpec(int(m["inner"]), int(m["state"]), int(m["dt_rank"]), int(m["conv"]))
+            elif l["type"] == "parallel":
+                mixer = ParallelSpec(cls._left(m["left"]), WkvSpec(int(m["right"]["heads"]), int(m["right"]["dim"])),
+                                     float(m.get("left_scale", 1.0)), float(m.get("right_scale", 1.0)))
+            else:
+                raise ValueError(f"Bibezen: unknown mixer type {l['type']!r}")
+            f = l.get("mlp")
+            mlp = None
+            if f is not None:
+                if f.get("kind") == "dense":
+                    mlp = ClampedFFSpec(int(f["ff"]), float(f["limit"]))
+                elif f.get("kind") == "moe":
+                    mlp = SoftmaxMoESpec(int(f["router"]["experts"]), int(f["router"]["top"]), int(f["expert"]["ff"]),
+                                         int((f.get("shared") or {}).get("ff", 0)))
+                    if not 1 <= mlp.top <= mlp.experts:
+                        raise ValueError("Bibezen: top must lie between 1 and the number of experts")
+                else:
+                    raise ValueError(f"Bibezen: unknown feed-forward kind {f.get('kind')!r}")
+            layers.append(LayerSpec(l["type"], mixer, mlp))
+        return cls(name=name, vocab_size=int(c["vocab"]), hidden_size=int(c["width"]), layers=tuple(layers),
+                   rms_eps=float(c["norm"]["eps"]), streams=int(c.get("streams") or 0),
+                   residual_mult=float(c.get("residual_mult", 1.0)),
+                   embed_scale=float((c.get("embedding") or {}).get("scale", 1.0)),
+                   canon_taps=int((c.get("canon") or {}).get("taps") or 0))
+
+    @classmethod
+    def uniform(cls, name: str, vocab: int, width: int, pattern: str, heads: int, kv_heads: int, dim: int, ff: int,
+                experts: int = 16, top: int = 2, expert_ff: int = 1536, streams: int = 2, window: int = 1024,
+                pool: int = 64, state: int = 16) -> "BibezenConfig":
+        """``pattern``: one letter per layer, W wkv / S selective scan / P parallel; upper case with
+        the mixture feed-forward (and a shared expert of ``expert_ff``), lower case with the dense one."""
+        layers = []
+        for ch in pattern:
+            up = ch.upper()
+            if up == "W":
+                mixer = WkvSpec(heads, dim)
+            elif up == "S":
+                mixer = SelectiveScanSpec(2 * width, state, max(width // 16, 1), 4)
+            else:
+                left = PooledWindowAttentionSpec(heads, kv_heads, dim, dim, dim ** -0.5, 30.0,
+                                                 RotarySpec(dim // 2, 1e6, None, True), window, pool, 4)
+                mixer = ParallelSpec(left, WkvSpec(heads, dim), 1.0, 1.0)
+            mlp = SoftmaxMoESpec(experts, top, expert_ff, expert_ff) if ch.isupper() else ClampedFFSpec(ff, 7.0)
+            layers.append(LayerSpec({"W": "wkv", "S": "mamba1", "P": "parallel"}[up], mixer, mlp))
+        return cls(name=name, vocab_size=vocab, hidden_size=width, layers=tuple(layers), rms_eps=1e-5, streams=streams,
+                   residual_mult=0.5, embed_scale=float(width) ** 0.5, canon_taps=3)
+
+
 # config.json "architecture" -> reader (checkpoints that are not HF Llama / Mixtral folders)
 ARCHITECTURES = {"Sapapel": SapapelConfig.from_json, "Kivezen": KivezenConfig.from_json,
-                 "Nopunex": NopunexConfig.from_json}
+                 "Nopunex": NopunexConfig.from_json, "Bibezen": BibezenConfig.from_json}
 
 PRESETS["tiny-sapapel"] = SapapelConfig.uniform("tiny-sapapel", 512, 128, 3, 4, 16, 32, 48, 64, 6, 2)
 # speed measurements (random weights): layer shapes of small production MoE models, and the
@@ -561,6 +761,14 @@ PRESETS["tiny-nopunex"] = NopunexConfig.uniform("tiny-nopunex", 512, 128, "AdMA"
 # feed-forwards of the MoE's active size
 PRESETS["nopunex-2k"] = NopunexConfig.uniform("nopunex-2k", 32000, 2048, "DAMADAMA", 16, 4, 128, 4608)
 PRESETS["nopunex-4k"] = NopunexConfig.uniform("nopunex-4k", 32000, 4096, "DAMA", 32, 8, 128, 6144)
+
+
+PRESETS["tiny-bibezen"] = BibezenConfig.uniform("tiny-bibezen", 512, 128, "wPSp", 4, 2, 32, 256, 6, 2, 64, window=40, pool=8)
+# speed measurements beside kivezen-2k / kivezen-4k (the closest family: fp32 hyper-connection
+# streams, a recurrent mixer among attention layers, a softmax-routed mixture with a shared expert):
+# the same width, depth, heads, KV heads, head size, experts and expert size
+PRESETS["bibezen-2k"] = BibezenConfig.uniform("bibezen-2k", 32000, 2048, "WPPPSPPP", 16, 4, 128, 4096, 16, 2, 1536)
+PRESETS["bibezen-4k"] = BibezenConfig.uniform("bibezen-4k", 32000, 4096, "WPSP", 32, 8, 128, 8192, 8, 2, 2048)
 
 
 def get_config(name_or_path: str):

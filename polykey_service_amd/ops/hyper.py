@@ -20,7 +20,7 @@ from . import gemm, native
 @dataclasses.dataclass
 class ExpertSum:
     """A mixture's output not yet summed: token t's y = sum_j wts[t, j] * y[inv[t * top + j]]
-    (+ sigmoid(gate[t]) * shared[t])."""
+    (+ sigmoid(gate[t]) * shared[t]; ``gate`` None: + shared[t])."""
     y: torch.Tensor                         # [n, W] expert rows in expert order
     inv: torch.Tensor                       # [T * top] int32 row of (token, choice); < 0: none
     wts: torch.Tensor                       # [T, top] fp32
@@ -33,7 +33,8 @@ class ExpertSum:
         rows = torch.where((idx >= 0)[..., None], self.y.float()[idx.clamp(min=0)], torch.zeros((), device=self.y.device))
         out = (rows * self.wts[..., None]).sum(1)
         if self.shared is not None:
-            out = out + self.shared.float() * torch.sigmoid(self.gate.float())[:, None]
+            out = out + (self.shared.float() * torch.sigmoid(self.gate.float())[:, None] if self.gate is not None
+                         else self.shared.float())
         return out
 
 
@@ -71,7 +72,7 @@ def hyper_step(xs: torch.Tensor, y, close: Optional[tuple], open_: Optional[tupl
     elif isinstance(y, ExpertSum):
         es, y = y, y.y
         assert es.inv.dtype == torch.int32 and es.wts.dtype == torch.float32 and es.wts.is_contiguous()
-        assert es.shared is None or (es.shared.is_contiguous() and es.gate.dtype == torch.float32)
+        assert es.shared is None or (es.shared.is_contiguous() and (es.gate is None or es.gate.dtype == torch.float32))
     assert y is None or y.is_contiguous()
     mix, a_out = close if close is not None else (None, None)
     a_in, w = open_ if open_ is not None else (None, None)
@@ -86,13 +87,14 @@ def hyper_step(xs: torch.Tensor, y, close: Optional[tuple], open_: Optional[tupl
     return act, z32
 
 
-def spread_rows(table: torch.Tensor, ids: torch.Tensor, S: int) -> torch.Tensor:
-    """xs[t, s] = table[ids[t]] as fp32 for every stream s: [T, S, W]."""
+def spread_rows(table: torch.Tensor, ids: torch.Tensor, S: int, scale: float = 1.0) -> torch.Tensor:
+    """xs[t, s] = table[ids[t]] * scale as fp32 for every stream s: [T, S, W]."""
     T, W = ids.numel(), table.shape[1]
     if not table.is_cuda:
-        return table[ids.long()].float()[:, None, :].repeat(1, S, 1)
+        rows = table[ids.long()].float()
+        return (rows if scale == 1.0 else rows * torch.tensor(scale, dtype=torch.float32))[:, None, :].repeat(1, S, 1)
     xs = torch.empty((T, S, W), dtype=torch.float32, device=table.device)
     assert table.is_contiguous() and ids.dtype == torch.int32
     native.call("pkm_spread_rows", xs.data_ptr(), table.data_ptr(), ids.data_ptr(), T, S, W, table.shape[0],
-                native.dt_code(table.dtype), native.stream_ptr())
+                native.dt_code(table.dtype), float(scale), native.stream_ptr())
     return xs

@@ -55,16 +55,23 @@ def _write_cache(cache: torch.Tensor, rows: torch.Tensor, slot_mapping: torch.Te
 
 def rotate_cache(proj: torch.Tensor, positions: torch.Tensor, slot_mapping: torch.Tensor, table: Optional[torch.Tensor],
                  halves: bool, k_cache: torch.Tensor, v_cache: torch.Tensor, QH: int, KH: int, VH: int, D: int,
-                 V: int) -> torch.Tensor:
+                 V: int, q_norm: Optional[torch.Tensor] = None, k_norm: Optional[torch.Tensor] = None,
+                 eps: float = 0.0) -> torch.Tensor:
     """proj [T, QH*D | KH*D | VH*V] (may be a column slice of a wider projection output): q and k
     heads turn by the token's position (``table`` rows; None: no rotation), k and v go to the paged
-    caches.  Returns q [T, QH, D] in the cache's dtype."""
+    caches.  ``q_norm`` / ``k_norm`` [D] fp32: the heads are first set to unit RMS (``eps`` inside
+    the root) times that weight.  Returns q [T, QH, D] in the cache's dtype."""
     T = proj.shape[0]
     q = torch.empty((T, QH, D), dtype=k_cache.dtype, device=proj.device)
     if not proj.is_cuda:
         f = proj.float()
         qq, kk = f[:, :QH * D].view(T, QH, D), f[:, QH * D:(QH + KH) * D].view(T, KH, D)
         vv = f[:, (QH + KH) * D:].view(T, VH, V)
+        unit = lambda u, w: u / torch.sqrt((u * u).mean(-1, keepdim=True) + eps) * w
+        if q_norm is not None:
+            qq = unit(qq, q_norm)
+        if k_norm is not None:
+            kk = unit(kk, k_norm)
         if table is not None:
             cs = table[positions.long()]
             qq, kk = turn(qq, cs, halves), turn(kk, cs, halves)
@@ -77,10 +84,13 @@ def rotate_cache(proj: torch.Tensor, positions: torch.Tensor, slot_mapping: torc
     assert k_cache.is_contiguous() and v_cache.is_contiguous()
     assert k_cache.shape[1:] == (KH, k_cache.shape[2], D) and v_cache.shape[1:] == (VH, k_cache.shape[2], V)
     assert table is None or (table.dtype == torch.float32 and table.is_contiguous() and 2 * table.shape[1] <= D)
+    for w in (q_norm, k_norm):
+        assert w is None or (w.dtype == torch.float32 and w.numel() == D)
     native.call("pkm_rotate_cache", q.data_ptr(), proj.data_ptr(), proj.stride(0), positions.data_ptr(),
                 slot_mapping.data_ptr(), native.ptr(table), table.shape[1] if table is not None else 0,
                 table.shape[0] if table is not None else 0, int(halves), k_cache.data_ptr(), v_cache.data_ptr(), T,
-                QH, KH, VH, D, V, k_cache.shape[2], native.dt_code(k_cache.dtype), native.stream_ptr())
+                QH, KH, VH, D, V, k_cache.shape[2], native.ptr(q_norm), native.ptr(k_norm), float(eps),
+                native.dt_code(k_cache.dtype), native.stream_ptr())
     return q
 
 
@@ -211,14 +221,17 @@ GATE_NONE, GATE_SIGMOID, GATE_SILU = 0, 1, 2
 
 def head_norm_gate(a: torch.Tensor, H: int, V: int, eps: float, gate: Optional[torch.Tensor], gate_kind: int,
                    dtype: torch.dtype, weight: Optional[torch.Tensor] = None, post: float = 1.0, pair_group: int = 0,
-                   coef: float = 0.0) -> torch.Tensor:
+                   coef: float = 0.0, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Per (token, head): u / sqrt(mean(u^2) + eps) * weight * post * act(gate) -> [T, H * V] in
     ``dtype``.  ``a`` fp32: [T, H, V] with u = a[t, h]; or with ``pair_group`` = r > 0 it is
     [T, 2H, V] laid out in groups of (r first maps, r second maps) and u = first - coef * second
     (head h = g r + j reads rows g 2r + j and g 2r + r + j).  ``gate`` [T, H * V] pre-activations
-    (may be a column slice), ``weight`` [V] fp32 shared by the heads or None."""
+    (may be a column slice), ``weight`` fp32 [V] shared by the heads, [H * V] one per head, or None.
+    ``out``: write there ([T, H * V], may be a column slice)."""
     T = a.shape[0]
-    out = torch.empty((T, H * V), dtype=dtype, device=a.device)
+    if out is None:
+        out = torch.empty((T, H * V), dtype=dtype, device=a.device)
+    per_head = weight is not None and weight.numel() == H * V and H > 1
     if not a.is_cuda:
         if pair_group:
             r = pair_group
@@ -228,7 +241,7 @@ def head_norm_gate(a: torch.Tensor, H: int, V: int, eps: float, gate: Optional[t
             u = a.view(T, H, V)
         z = u / torch.sqrt((u * u).mean(-1, keepdim=True) + eps) * post
         if weight is not None:
-            z = z * weight
+            z = z * (weight.view(H, V) if per_head else weight)
         z = z.reshape(T, H * V)
         if gate_kind == GATE_SIGMOID:
             z = z * torch.sigmoid(gate.float())
@@ -237,9 +250,10 @@ def head_norm_gate(a: torch.Tensor, H: int, V: int, eps: float, gate: Optional[t
         out.copy_(z)
         return out
     assert a.dtype == torch.float32 and a.is_contiguous() and (gate is None or gate.stride(1) == 1)
-    assert weight is None or (weight.dtype == torch.float32 and weight.numel() == V)
-    native.call("pkm_head_norm_gate", out.data_ptr(), a.data_ptr(), T, H, V, float(eps), native.ptr(gate),
+    assert weight is None or (weight.dtype == torch.float32 and weight.numel() in (V, H * V))
+    assert out.stride(1) == 1 and out.shape == (T, H * V)
+    native.call("pkm_head_norm_gate", out.data_ptr(), out.stride(0), a.data_ptr(), T, H, V, float(eps), native.ptr(gate),
                 gate.stride(0) if gate is not None else 0, native.dt_code(gate.dtype) if gate is not None else 1,
-                int(gate_kind if gate is not None else GATE_NONE), native.ptr(weight), float(post), int(pair_group),
-                float(coef), native.dt_code(dtype), native.stream_ptr())
+                int(gate_kind if gate is not None else GATE_NONE), native.ptr(weight), V if per_head else 0, float(post),
+                int(pair_group), float(coef), native.dt_code(out.dtype), native.stream_ptr())
     return out

@@ -433,3 +433,48 @@ def clamped_experts(x_act: torch.Tensor, ids: torch.Tensor, gate, up, down, limi
                 offsets.data_ptr(), sorted_.data_ptr(), float(limit), n, k, E, F_, W, dt, st)
     native.call("pkm_expert_down", y.data_ptr(), h.data_ptr(), down.data_ptr(), offsets.data_ptr(), n, E, W, F_, dt, st)
     return y, inv
+
+
+def silu_experts(x_act: torch.Tensor, ids: torch.Tensor, gate, up, down, w13=None, w2=None, w13_p=None, w2_p=None):
+    """Rows of every (token, chosen expert) pair through down_e(silu(gate_e x) * (up_e x)): (y [T * top, W]
+    in expert order, inv [T * top]) for the kernel that sums them with the routing weights.  With
+    ``w13`` / ``w2`` (shapes of :func:`mfma_experts_ok`) the framework's grouped MFMA GEMMs with the
+    fused SiLU epilogue, else gate / up [E, F, W], down [E, W, F] through the tiled FMA grouped
+    kernels (any sizes, fp32 too)."""
+    T, W = x_act.shape
+    k = ids.shape[1]
+    n = T * k
+    if w13 is not None:
+        E = w13.shape[0]
+        offsets, sorted_, inv = align(ids, E, 0, E)
+        if T <= 64 and E <= 64 and gemm.SKINNY_ENABLED:  # decode: the GEMM gathers the tokens' rows itself
+            h = gemm.grouped_linear(x_act, w13, offsets, T, True, packed=w13_p, a_rows=sorted_, a_row_div=k, n_rows=n)
+            return gemm.grouped_linear(h, w2, offsets, T, False, packed=w2_p), inv
+        xs = permute(x_act, sorted_, offsets, k)
+        h = grouped_gemm(xs, w13, offsets, T, silu=True, packed=w13_p)
+        return grouped_gemm(h, w2, offsets, T, silu=False, packed=w2_p), inv
+    E, F_, _ = gate.shape
+    offsets, sorted_, inv = align(ids, E, 0, E)
+    if not x_act.is_cuda:
+        m = int(offsets[-1])
+        tok = sorted_[:m].long() // k
+        y = torch.zeros((m, W), dtype=torch.float32)
+        offs = offsets.tolist()
+        for e in range(E):
+            lo, hi = offs[e], offs[e + 1]
+            if hi > lo:
+                xe = x_act[tok[lo:hi]]
+                g = F.linear(xe, gate[e]).float()
+                h = (g * torch.sigmoid(g) * F.linear(xe, up[e]).float()).to(x_act.dtype)
+                y[lo:hi] = F.linear(h, down[e]).float()
+        return y, inv
+    assert x_act.is_contiguous() and gate.is_contiguous() and up.is_contiguous() and down.is_contiguous()
+    dt = native.dt_code(x_act.dtype)
+    h = torch.empty((n, F_), dtype=x_act.dtype, device=x_act.device)
+    y = torch.empty((n, W), dtype=torch.float32, device=x_act.device)
+    st = native.stream_ptr()
+    # limit 0 selects the unclamped SiLU product in the grouped kernel's epilogue
+    native.call("pkm_expert_gate_up_clamped", h.data_ptr(), x_act.data_ptr(), gate.data_ptr(), up.data_ptr(),
+                offsets.data_ptr(), sorted_.data_ptr(), 0.0, n, k, E, F_, W, dt, st)
+    native.call("pkm_expert_down", y.data_ptr(), h.data_ptr(), down.data_ptr(), offsets.data_ptr(), n, E, W, F_, dt, st)
+    return y, inv

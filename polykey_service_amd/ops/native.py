@@ -87,7 +87,7 @@ MIXER_SIGNATURES = {
     "pkm_permute_scaled": [P, P, P, P, I32, I32, I32, I32, P],
     "pkm_expert_align_wide": [P, P, P, P, I32, I32, P],
     "pkm_expert_gate_up_clamped": [P, P, P, P, P, P, F32, I32, I32, I32, I32, I32, I32, P],
-    "pkm_spread_rows": [P, P, P, I32, I32, I32, I32, I32, P],
+    "pkm_spread_rows": [P, P, P, I32, I32, I32, I32, I32, F32, P],
     "pkm_hyper_step": [P, I32, I32, I32, P, I32, I32, P, I32, P, P, I32, P, I64, P, P, P, P, F32, P, I32, P, P, P],
     "pkm_tanh_cap": [P, I64, F32, P],
     "pkm_route_topk_softmax": [P, P, P, I64, I32, I32, I32, P],
@@ -104,18 +104,27 @@ MIXER_SIGNATURES = {
     "pkm_join_cast": [P, P, P, I32, I32, I32, P],
     "pkm_silu_mul": [P, P, I32, I32, I32, I32, I32, P],
     "pkm_scale": [P, I64, F32, P],
-    "pkm_rotate_cache": [P, P, I64, P, P, P, I32, I32, I32, P, P, I32, I32, I32, I32, I32, I32, I32, I32, P],
+    "pkm_rotate_cache": [P, P, I64, P, P, P, I32, I32, I32, P, P, I32, I32, I32, I32, I32, I32, I32, P, P, F32, I32, P],
     "pkm_latent_in": [P, P, P, I64, I32, I32, I32, P, P, F32, P, P, P, I32, I32, I32, I32, I32, I32, P],
     "pkm_latent_query": [P, P, P, P, P, I32, I32, I32, I32, I32, I32, I32, I32, I32, P],
     "pkm_masked_attention": [P, I64, I64, I32, P, I32, P, P, I32, P, I64, P, P, P, I32, I32, I32, I32, I32, I32, I32, I32,
                              F32, I32, I32, I32, P, P, I32, I32, I32, P],
     "pkm_masked_decode_part": [I32, I32, I32, I32, I32, I32, I32, I32, I32, I32, I32],
     "pkm_set_masked_mfma": [I32],
-    "pkm_head_norm_gate": [P, P, I32, I32, I32, F32, P, I64, I32, I32, P, F32, I32, F32, I32, P],
+    "pkm_head_norm_gate": [P, I64, P, I32, I32, I32, F32, P, I64, I32, I32, P, I32, F32, I32, F32, I32, P],
     "pkm_conv_unit": [P, P, I64, P, I32, P, P, P, P, P, I32, I32, I32, I32, I32, I32, I32, P],
     "pkm_delta_rule": [P, P, P, I64, I32, P, P, P, P, P, P, I32, I32, I32, I32, I32, I32, P],
     "pkm_sink_attention": [P, P, P, P, P, I64, P, P, P, P, P, I32, I32, I32, I32, I32, I32, I32, I32, F32, F32, I32,
                            P, P, I32, I32, I32, P],
+    "pkm_causal_conv": [P, I32, P, I32, I64, P, P, I32, P, P, P, P, P, P, I32, I32, I32, I32, I32, P],
+    "pkm_shift_mix": [P, P, P, I32, P, P, P, P, P, I32, I32, I32, I32, P],
+    "pkm_tanh": [P, I64, I32, P],
+    "pkm_wkv": [P, P, I64, P, P, P, P, P, P, P, I32, I32, I32, I32, I32, P],
+    "pkm_selective_scan": [P, P, I64, P, I64, P, P, P, I64, P, P, I64, P, P, P, P, I32, I32, I32, I32, I32, P],
+    "pkm_pool_update": [P, P, P, P, P, P, P, I64, I32, I32, I32, I32, I32, I32, I32, P],
+    "pkm_pooled_attention": [P, P, P, P, P, P, P, I64, P, P, P, I32, I32, I32, I32, I32, I32, I32, F32, F32, I32, I32, I32,
+                             I32, P],
+    "pkm_mix_heads": [P, I64, I32, P, P, I32, I32, I32, I32, F32, P],
 }
 _mixers: Optional[ctypes.CDLL] = None
 
