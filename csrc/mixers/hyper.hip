@@ -1,9 +1,9 @@
 // Residual streams of pre-norm layers, kept in fp32, one or several per token (hyper-connections).
 //
-//   spread_rows   xs[t, s] = table[ids[t]] for every stream s
+//   spread_rows   xs[t, s] = table[ids[t]] * scale for every stream s
 //   hyper_step    closes one sublayer and opens the next, per token, in one pass:
 //                   y      = the sublayer's output row: a plain row, the sum of split-K slabs, or a
-//                            mixture's  sum_j wts[t, j] * rows[inv[t, j]]  (+ sigmoid(gate[t]) * shared[t])
+//                            mixture's  sum_j wts[t, j] * rows[inv[t, j]]  (+ [sigmoid(gate[t]) *] shared[t])
 //                   xs'[t] = sum_s mix[s, t] xs[s] + a_out[t] y          (all streams from the old ones)
 //                   u      = sum_t a_in[t] xs'[t];  z = u / sqrt(mean(u^2) + eps) * w
 //                 either half may be absent; with `rows` only those tokens are opened (the rows whose
@@ -22,14 +22,15 @@ constexpr int kMaxStreams = 8;
 
 template <typename T>
 __global__ void __launch_bounds__(256) spread_rows_kernel(float* __restrict__ xs, const T* __restrict__ table,
-                                                          const int* __restrict__ ids, int S, int W, int vocab) {
+                                                          const int* __restrict__ ids, int S, int W, int vocab,
+                                                          float scale) {
   const int t = blockIdx.x;
   int id = ids[t];
   id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
   const T* src = table + static_cast<int64_t>(id) * W;
   float* dst = xs + static_cast<int64_t>(t) * S * W;
   for (int i = threadIdx.x; i < W; i += blockDim.x) {
-    const float v = ld<T>(src + i);
+    const float v = ld<T>(src + i) * scale;
     for (int s = 0; s < S; ++s) dst[s * W + i] = v;
   }
 }
@@ -107,7 +108,7 @@ __global__ void __launch_bounds__(1024) hyper_step_kernel(HyperArgs a) {
   __syncthreads();
   const Y* y = static_cast<const Y*>(a.y);
   const T* y2 = static_cast<const T*>(a.y2);
-  const float gate = y2 ? sigmoidf(a.g2[src * a.g2_stride]) : 0.f;
+  const float gate = y2 ? (a.g2 ? sigmoidf(a.g2[src * a.g2_stride]) : 1.f) : 0.f;
   float ss = 0.f;
   float4 ur[NG];
   if (VEC >= 4) {
@@ -225,17 +226,17 @@ __global__ void __launch_bounds__(256) tanh_cap_kernel(float* __restrict__ x, in
 }  // namespace
 
 PK_EXPORT int pkm_spread_rows(void* xs, const void* table, const void* ids, int T, int S, int W, int vocab, int dt,
-                              hipStream_t stream) {
+                              float scale, hipStream_t stream) {
   if (T <= 0) return 0;
   if (S < 1 || S > kMaxStreams) return -1;
   PKM_DISPATCH(dt, E, spread_rows_kernel<E><<<T, 256, 0, stream>>>(static_cast<float*>(xs), static_cast<const E*>(table),
-                                                                    static_cast<const int*>(ids), S, W, vocab));
+                                                                    static_cast<const int*>(ids), S, W, vocab, scale));
   return PK_CHECK_LAUNCH();
 }
 
 // xs [tokens, S, W] fp32, updated in place when mix / a_out are given (then y, or inv / wts / y rows,
 // is the sublayer output; y_dt its element type, -1: none).  y2 / g2: a second row per token in the
-// activation type and its pre-sigmoid gate (fp32, element stride g2_stride).  a_in / norm_w: open.
+// activation type and its pre-sigmoid gate (fp32, element stride g2_stride; null: the row is added as it is).  a_in / norm_w: open.
 // rows: R token indices to open (no close).  act (element type act_dt) and z32 may each be null.
 PK_EXPORT int pkm_hyper_step(void* xs, int R, int S, int W, const void* y, int y_dt, int nslab, const void* inv, int top,
                              const void* wts, const void* y2, int y2_dt, const void* g2, long long g2_stride,
@@ -246,7 +247,7 @@ PK_EXPORT int pkm_hyper_step(void* xs, int R, int S, int W, const void* y, int y
   if ((mix == nullptr) != (a_out == nullptr) || (a_in == nullptr) != (norm_w == nullptr)) return -1;
   if (rows && mix) return -1;
   if (inv && (!y || !wts || top < 1 || nslab > 1)) return -1;
-  if (y2 && (!g2 || y2_dt != act_dt)) return -1;
+  if (y2 && y2_dt != act_dt) return -1;
   HyperArgs a{static_cast<float*>(xs), S, W, y, nslab, static_cast<int64_t>(R) * W, static_cast<const int*>(inv), top,
               static_cast<const float*>(wts), y2, static_cast<const float*>(g2), g2_stride,
               static_cast<const float*>(mix), static_cast<const float*>(a_out), static_cast<const float*>(a_in),

@@ -30,16 +30,35 @@ __device__ __forceinline__ int clamp_pos(int pos, int rows) { return pos < 0 ? 0
 
 // one wave turns one head: x[i], x[i + pairs] (halves) or x[2i], x[2i + 1] of the first 2 * pairs
 // coordinates by (cos, sin) = cs[2i], cs[2i + 1]; the rest pass.  IN -> OUT element types.
+// nw [D] fp32 or null: the head is first set to unit RMS (eps inside the root) times that weight.
 template <typename IN, typename OUT>
-__device__ __forceinline__ void turn_head(OUT* dst, const IN* src, int D, const float* cs, int pairs, int halves, int lane) {
+__device__ __forceinline__ void turn_head(OUT* dst, const IN* src, int D, const float* cs, int pairs, int halves, int lane,
+                                          const float* nw = nullptr, float eps = 0.f) {
+  float k = 1.f;
+  if (nw) {
+    float ss = 0.f;
+    for (int i = lane; i < D; i += 64) {
+      const float x = ld<IN>(src + i);
+      ss += x * x;
+    }
+    ss = pk::wave_sum(ss);
+    k = 1.f / sqrtf(ss / static_cast<float>(D) + eps);
+  }
   for (int i = lane; i < pairs; i += 64) {
     const int iu = halves ? i : 2 * i, iv = halves ? i + pairs : 2 * i + 1;
-    const float u = ld<IN>(src + iu), v = ld<IN>(src + iv);
+    float u = ld<IN>(src + iu), v = ld<IN>(src + iv);
+    if (nw) {
+      u = u * k * nw[iu];
+      v = v * k * nw[iv];
+    }
     const float c = cs[2 * i], s = cs[2 * i + 1];
     st<OUT>(dst + iu, u * c - v * s);
     st<OUT>(dst + iv, v * c + u * s);
   }
-  for (int i = 2 * pairs + lane; i < D; i += 64) st<OUT>(dst + i, ld<IN>(src + i));
+  for (int i = 2 * pairs + lane; i < D; i += 64) {
+    const float x = ld<IN>(src + i);
+    st<OUT>(dst + i, nw ? x * k * nw[i] : x);
+  }
 }
 
 template <typename T>
@@ -47,7 +66,7 @@ __global__ void __launch_bounds__(64)
 rotate_cache_kernel(T* __restrict__ q_out, const T* __restrict__ proj, int64_t stride, const int* __restrict__ positions,
                     const int* __restrict__ slot_mapping, const float* __restrict__ table, int pairs, int table_rows,
                     int halves, T* __restrict__ k_cache, T* __restrict__ v_cache, int QH, int KH, int VH, int D, int V,
-                    int bs) {
+                    int bs, const float* __restrict__ q_norm, const float* __restrict__ k_norm, float eps) {
   const int t = blockIdx.x, item = blockIdx.y, lane = threadIdx.x;
   const int slot = slot_mapping[t];
   const T* row = proj + static_cast<int64_t>(t) * stride;
@@ -55,12 +74,12 @@ rotate_cache_kernel(T* __restrict__ q_out, const T* __restrict__ proj, int64_t s
   const int np = cs ? pairs : 0;
   if (item < QH) {
     turn_head<T, T>(q_out + (static_cast<int64_t>(t) * QH + item) * D, row + static_cast<int64_t>(item) * D, D, cs, np,
-                    halves, lane);
+                    halves, lane, q_norm, eps);
   } else if (item < QH + KH) {
     if (slot < 0) return;
     const int g = item - QH;
     turn_head<T, T>(k_cache + ((static_cast<int64_t>(slot / bs) * KH + g) * bs + slot % bs) * D,
-                    row + static_cast<int64_t>(item) * D, D, cs, np, halves, lane);
+                    row + static_cast<int64_t>(item) * D, D, cs, np, halves, lane, k_norm, eps);
   } else {
     if (slot < 0) return;
     const int g = item - QH - KH;
@@ -637,9 +656,9 @@ constexpr int kGateNone = 0, kGateSigmoid = 1, kGateSilu = 2;
 // one wave per (token, head)
 template <typename GT, typename OT>
 __global__ void __launch_bounds__(64)
-head_norm_gate_kernel(OT* __restrict__ out, const float* __restrict__ a, int H, int V, float eps, const GT* __restrict__ gate,
-                      int64_t gate_stride, int gate_kind, const float* __restrict__ weight, float post, int pair_group,
-                      float coef) {
+head_norm_gate_kernel(OT* __restrict__ out, int64_t out_stride, const float* __restrict__ a, int H, int V, float eps,
+                      const GT* __restrict__ gate, int64_t gate_stride, int gate_kind, const float* __restrict__ weight,
+                      int weight_hs, float post, int pair_group, float coef) {
   const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const float *u1, *u2 = nullptr;
   if (pair_group > 0) {
@@ -656,7 +675,8 @@ head_norm_gate_kernel(OT* __restrict__ out, const float* __restrict__ a, int H, 
   }
   ss = pk::wave_sum(ss);
   const float k = post / sqrtf(ss / static_cast<float>(V) + eps);
-  OT* dst = out + (static_cast<int64_t>(t) * H + h) * V;
+  OT* dst = out + static_cast<int64_t>(t) * out_stride + static_cast<int64_t>(h) * V;
+  if (weight) weight += static_cast<int64_t>(h) * weight_hs;
   const GT* gr = gate ? gate + static_cast<int64_t>(t) * gate_stride + static_cast<int64_t>(h) * V : nullptr;
   for (int i = lane; i < V; i += 64) {
     float z = (u2 ? u1[i] - coef * u2[i] : u1[i]) * k;
@@ -671,18 +691,20 @@ head_norm_gate_kernel(OT* __restrict__ out, const float* __restrict__ a, int H, 
 
 }  // namespace
 
-// proj [T, QH*D | KH*D | VH*V] rows `stride` elements apart; table [table_rows, pairs, 2] fp32 or null
+// proj [T, QH*D | KH*D | VH*V] rows `stride` elements apart; table [table_rows, pairs, 2] fp32 or null;
+// q_norm / k_norm [D] fp32 or null: unit RMS times the weight before the rotation
 PK_EXPORT int pkm_rotate_cache(void* q_out, const void* proj, long long stride, const void* positions,
                                const void* slot_mapping, const void* table, int pairs, int table_rows, int halves,
-                               void* k_cache, void* v_cache, int T, int QH, int KH, int VH, int D, int V, int bs, int dt,
-                               hipStream_t stream) {
+                               void* k_cache, void* v_cache, int T, int QH, int KH, int VH, int D, int V, int bs,
+                               const void* q_norm, const void* k_norm, float eps, int dt, hipStream_t stream) {
   if (T <= 0) return 0;
   if (D < 1 || V < 1 || 2 * pairs > D || (table && table_rows < 1) || bs < 1) return -1;
   const dim3 grid(T, QH + KH + VH);
   PKM_DISPATCH(dt, E, rotate_cache_kernel<E><<<grid, 64, 0, stream>>>(
                           static_cast<E*>(q_out), static_cast<const E*>(proj), stride, static_cast<const int*>(positions),
                           static_cast<const int*>(slot_mapping), static_cast<const float*>(table), pairs, table_rows,
-                          halves, static_cast<E*>(k_cache), static_cast<E*>(v_cache), QH, KH, VH, D, V, bs));
+                          halves, static_cast<E*>(k_cache), static_cast<E*>(v_cache), QH, KH, VH, D, V, bs,
+                          static_cast<const float*>(q_norm), static_cast<const float*>(k_norm), eps));
   return PK_CHECK_LAUNCH();
 }
 
@@ -798,17 +820,20 @@ PK_EXPORT int pkm_set_masked_mfma(int on) {
 }
 
 // a fp32 [T, H, V] (pair_group = 0) or [T, 2H, V] in groups of (r first maps, r second maps);
-// gate [T, H * V] rows gate_stride elements apart (gate_dt) or null; weight [V] fp32 or null
-PK_EXPORT int pkm_head_norm_gate(void* out, const void* a, int T, int H, int V, float eps, const void* gate,
-                                 long long gate_stride, int gate_dt, int gate_kind, const void* weight, float post,
-                                 int pair_group, float coef, int out_dt, hipStream_t stream) {
+// gate [T, H * V] rows gate_stride elements apart (gate_dt) or null; weight fp32 or null, head h reads
+// weight[h * weight_hs ...] (0: one [V] for all heads); out rows out_stride elements apart
+PK_EXPORT int pkm_head_norm_gate(void* out, long long out_stride, const void* a, int T, int H, int V, float eps,
+                                 const void* gate, long long gate_stride, int gate_dt, int gate_kind, const void* weight,
+                                 int weight_hs, float post, int pair_group, float coef, int out_dt, hipStream_t stream) {
   if (T <= 0) return 0;
-  if (H < 1 || V < 1 || pair_group < 0 || (pair_group > 0 && H % pair_group)) return -1;
+  if (H < 1 || V < 1 || pair_group < 0 || (pair_group > 0 && H % pair_group) || out_stride < static_cast<long long>(H) * V)
+    return -1;
   const dim3 grid(T, H);
 #define PKM_HNG(GT)                                                                                                  \
   PKM_DISPATCH(out_dt, O, head_norm_gate_kernel<GT, O><<<grid, 64, 0, stream>>>(                                       \
-                              static_cast<O*>(out), static_cast<const float*>(a), H, V, eps, static_cast<const GT*>(gate), \
-                              gate_stride, gate_kind, static_cast<const float*>(weight), post, pair_group, coef))
+                              static_cast<O*>(out), out_stride, static_cast<const float*>(a), H, V, eps,             \
+                              static_cast<const GT*>(gate), gate_stride, gate_kind, static_cast<const float*>(weight),   \
+                              weight_hs, post, pair_group, coef))
   if (gate_dt == kF32) {
     PKM_HNG(float);
   } else if (gate_dt == kBF16) {

@@ -1,0 +1,334 @@
+// Sliding-window softmax attention over a paged cache that also sees block means of the keys and
+// values behind the window, with capped scores, sink logits and mixing of the heads' weights.
+//
+//   pool_update        for a token at the last position of a block of `pool`: the mean of the block's
+//                      cached key / value rows goes to entry position / pool of the mean caches
+//   pooled_attention   query at position p sees single keys max(0, p - window + 1) <= j <= p and the
+//                      means of blocks b < floor((p - window + 1) / pool);  s = cap tanh(q . k scale / cap);
+//                      p_j = exp(s_j) / (exp(sink_h) + sum exp(s_j')) over both kinds of keys;
+//                      out[t, h, g] = sum_j p_j v_(g, j) for every value head g (all_values) or the own one
+//   mix_heads          out[t, h] = post * sum_g talk[h, g] o[t, g, value head of h]
+//
+// Scores, softmax, means and sums are fp32 for both element types.  The (token, head) pairs of a
+// sequence that share a key head are the rows of one tile problem against key / value tiles staged
+// once in LDS; the tiles of the means and of the single keys each start at multiples of the tile
+// size counted from entry 0 of the sequence, so a position's sums run in the same order however its
+// prompt was cut and whatever else the step holds.
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+
+#include "mix_common.h"
+
+using namespace pkm;
+
+namespace {
+
+// one workgroup per (token, key head): thread c sums column c of the block's rows in position order
+template <typename T>
+__global__ void __launch_bounds__(256)
+pool_update_kernel(const T* __restrict__ k_cache, const T* __restrict__ v_cache, T* __restrict__ kp_cache,
+                   T* __restrict__ vp_cache, const int* __restrict__ positions, const int* __restrict__ token_seq,
+                   const int* __restrict__ block_tables, int64_t bt_stride, int G, int D, int V, int bs, int pool) {
+  const int t = blockIdx.x, g = blockIdx.y;
+  const int pos = positions[t];
+  if (pos < 0 || (pos + 1) % pool != 0) return;
+  const int* bt = block_tables + static_cast<int64_t>(token_seq[t]) * bt_stride;
+  const int b = pos / pool;
+  const int64_t dst = (static_cast<int64_t>(bt[b / bs]) * G + g) * bs + b % bs;
+  const float inv = 1.f / static_cast<float>(pool);
+  for (int c = threadIdx.x; c < D + V; c += 256) {
+    const bool key = c < D;
+    const T* src = key ? k_cache : v_cache;
+    const int w = key ? D : V, cc = key ? c : c - D;
+    float acc = 0.f;
+    for (int j = pos - pool + 1; j <= pos; ++j)
+      acc += ld<T>(src + ((static_cast<int64_t>(bt[j / bs]) * G + g) * bs + j % bs) * w + cc);
+    st<T>((key ? kp_cache : vp_cache) + dst * w + cc, acc * inv);
+  }
+}
+
+constexpr int kBQ = 16;        // (token, head) rows per workgroup
+constexpr int kThreads = 256;  // 16 rows x 16 lanes
+
+struct PooledArgs {
+  float* out;  // [T, H, VG, V]
+  const void* q;  // [T, H, D]
+  const void *k_cache, *v_cache, *kp_cache, *vp_cache;  // [blocks, G, bs, D | V]
+  const int* block_tables;
+  int64_t bt_stride;
+  const int* cu_q;
+  const int* context_lens;
+  const float* sink;  // [H] logits or null
+  int n_seqs, H, G, D, V, bs, BK;
+  float scale, softcap;
+  int window, pool, all_values;
+};
+
+__device__ __forceinline__ int blocks_seen(int pos, int window, int pool) {
+  if (window <= 0 || pool <= 0) return 0;
+  const int n = pos - window + 1;
+  return n >= pool ? n / pool : 0;
+}
+
+// NV: output accumulators per thread = ceil(value columns / 16)
+template <typename T, int NV>
+__global__ void __launch_bounds__(kThreads) pooled_attention_kernel(PooledArgs a) {
+  extern __shared__ float smem[];
+  const int H = a.H, G = a.G, D = a.D, V = a.V, BK = a.BK, bs = a.bs;
+  const int R = H / G;
+  const int kh = blockIdx.y;
+  const int VG = a.all_values ? G : 1;
+  const int VW = VG * V;  // value columns staged per key
+  int s = 0, tile = blockIdx.x;
+  for (; s < a.n_seqs; ++s) {
+    const int rows = (a.cu_q[s + 1] - a.cu_q[s]) * R;
+    const int nt = (rows + kBQ - 1) / kBQ;
+    if (tile < nt) break;
+    tile -= nt;
+  }
+  if (s >= a.n_seqs) return;
+  const int q0 = a.cu_q[s], qlen = a.cu_q[s + 1] - q0, ctx = a.context_lens[s];
+  const int n_rows = qlen * R;
+  const int row0 = tile * kBQ;
+  const int DS = D + 1, VS = VW + 1;  // odd row strides: conflict-free column walks
+  float* qs = smem;             // [kBQ][DS]
+  float* ks = qs + kBQ * DS;    // [BK][DS]
+  float* vs = ks + BK * DS;     // [BK][VS]
+  float* ps = vs + BK * VS;     // [kBQ][BK]
+  float* m_s = ps + kBQ * BK;   // [kBQ] running max
+  float* l_s = m_s + kBQ;       // [kBQ] running sum
+  const int tid = threadIdx.x;
+  const int qi = tid >> 4, kg = tid & 15;
+  const int* bt = a.block_tables + static_cast<int64_t>(s) * a.bt_stride;
+
+  for (int e = tid; e < kBQ * D; e += kThreads) {
+    const int r = e / D, c = e - r * D;
+    const int row = row0 + r;
+    float v = 0.f;
+    if (row < n_rows) {
+      const int tl = row / R, h = kh * R + row - tl * R;
+      v = ld<T>(static_cast<const T*>(a.q) + (static_cast<int64_t>(q0 + tl) * H + h) * D + c);
+    }
+    qs[r * DS + c] = v;
+  }
+  const int my_row = row0 + qi;
+  const bool live = my_row < n_rows;
+  const int my_tl = live ? my_row / R : 0;
+  const int my_h = kh * R + (live ? my_row - my_tl * R : 0);
+  const int my_pos = live ? ctx - qlen + my_tl : -1;
+  const int my_lo = (live && a.window > 0) ? max(0, my_pos - a.window + 1) : 0;
+  const int my_blocks = live ? blocks_seen(my_pos, a.window, a.pool) : 0;
+  if (tid < kBQ) {
+    const int row = row0 + tid;
+    const int h = kh * R + (row < n_rows ? row % R : 0);
+    m_s[tid] = a.sink ? a.sink[h] : -INFINITY;  // the sink is a key without a value
+    l_s[tid] = a.sink ? 1.f : 0.f;
+  }
+  const int first_pos = ctx - qlen + row0 / R;
+  const int last_pos = ctx - qlen + (min(row0 + kBQ, n_rows) - 1) / R;
+  float acc[NV];
+#pragma unroll
+  for (int i = 0; i < NV; ++i) acc[i] = 0.f;
+  __syncthreads();
+
+  // part 0: the block means (entries [0, blocks seen by the tile's last row)); part 1: single keys
+  for (int part = 0; part < 2; ++part) {
+    const T* kc = static_cast<const T*>(part ? a.k_cache : a.kp_cache);
+    const T* vc = static_cast<const T*>(part ? a.v_cache : a.vp_cache);
+    int k_begin, k_end;
+    if (part == 0) {
+      k_begin = 0;
+      k_end = last_pos >= 0 ? blocks_seen(last_pos, a.window, a.pool) : 0;
+    } else {
+      k_end = last_pos + 1;
+      k_begin = (first_pos >= 0 && a.window > 0) ? max(0, first_pos - a.window + 1) / BK * BK : 0;
+    }
+    for (int k0 = k_begin; k0 < k_end; k0 += BK) {
+      const int nk = min(BK, k_end - k0);
+      for (int e = tid; e < BK * D; e += kThreads) {
+        const int j = e / D, c = e - j * D;
+        float v = 0.f;
+        if (j < nk) {
+          const int key = k0 + j;
+          v = ld<T>(kc + ((static_cast<int64_t>(bt[key / bs]) * G + kh) * bs + key % bs) * D + c);
+        }
+        ks[j * DS + c] = v;
+      }
+      for (int e = tid; e < BK * VW; e += kThreads) {
+        const int j = e / VW, c = e - j * VW;
+        float v = 0.f;
+        if (j < nk) {
+          const int key = k0 + j;
+          const int g = a.all_values ? c / V : kh, cc = a.all_values ? c - g * V : c;
+          v = ld<T>(vc + ((static_cast<int64_t>(bt[key / bs]) * G + g) * bs + key % bs) * V + cc);
+        }
+        vs[j * VS + c] = v;
+      }
+      __syncthreads();
+      float tmax = -INFINITY;
+      for (int j = kg; j < BK; j += 16) {
+        float d = 0.f;
+        const float* qr = qs + qi * DS;
+        const float* kr = ks + j * DS;
+        for (int c = 0; c < D; ++c) d += qr[c] * kr[c];
+        d *= a.scale;
+        if (a.softcap > 0.f) d = a.softcap * tanhf(d / a.softcap);
+        const int key = k0 + j;
+        const bool seen = part == 0 ? key < my_blocks : (key <= my_pos && key >= my_lo);
+        d = (j < nk && seen) ? d : -INFINITY;
+        ps[qi * BK + j] = d;
+        tmax = fmaxf(tmax, d);
+      }
+#pragma unroll
+      for (int o = 8; o > 0; o >>= 1) tmax = fmaxf(tmax, __shfl_xor(tmax, o, 64));
+      const float m_old = m_s[qi];
+      const float m_new = fmaxf(m_old, tmax);
+      float tsum = 0.f;
+      for (int j = kg; j < BK; j += 16) {
+        const float sc = ps[qi * BK + j];
+        const float p = (m_new == -INFINITY || sc == -INFINITY) ? 0.f : expf(sc - m_new);
+        ps[qi * BK + j] = p;
+        tsum += p;
+      }
+#pragma unroll
+      for (int o = 8; o > 0; o >>= 1) tsum += __shfl_xor(tsum, o, 64);
+      const float resc = (m_old == -INFINITY) ? 0.f : expf(m_old - m_new);
+      __syncthreads();  // every lane of the row has read m_old and its own scores
+      if (kg == 0) {
+        m_s[qi] = m_new;
+        l_s[qi] = l_s[qi] * resc + tsum;
+      }
+#pragma unroll
+      for (int i = 0; i < NV; ++i) acc[i] *= resc;
+      for (int j = 0; j < nk; ++j) {
+        const float p = ps[qi * BK + j];
+        const float* vr = vs + j * VS + kg;
+#pragma unroll
+        for (int i = 0; i < NV; ++i)
+          if (kg + 16 * i < VW) acc[i] += p * vr[16 * i];
+      }
+      __syncthreads();
+    }
+  }
+  const float l = l_s[qi];
+  const float inv = l > 0.f ? 1.f / l : 0.f;
+  if (!live) return;
+  float* dst = a.out + (static_cast<int64_t>(q0 + my_tl) * H + my_h) * VW;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int c = kg + 16 * i;
+    if (c < VW) dst[c] = acc[i] * inv;
+  }
+}
+
+size_t lds_bytes(int D, int VW, int bk) {
+  return (static_cast<size_t>(kBQ) * (D + 1) + static_cast<size_t>(bk) * (D + 1 + VW + 1) + kBQ * bk + 2 * kBQ) * 4;
+}
+
+// key tile: the largest of 64 / 32 / 16 whose tiles fit 60 KiB of LDS, else the largest of 32 / 16 / 8
+// within 144 KiB; 0: the heads are too wide
+int key_tile(int D, int VW) {
+  for (int bk = 64; bk >= 16; bk >>= 1)
+    if (lds_bytes(D, VW, bk) <= 60 * 1024) return bk;
+  for (int bk = 32; bk >= 8; bk >>= 1)
+    if (lds_bytes(D, VW, bk) <= 144 * 1024) return bk;
+  return 0;
+}
+
+template <typename T, int NV>
+int launch_one(const PooledArgs& a, dim3 grid, size_t lds, hipStream_t stream) {
+  if (lds > 60 * 1024) {
+    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(pooled_attention_kernel<T, NV>),
+                                             hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));
+    if (e != hipSuccess) return static_cast<int>(e);
+  }
+  pooled_attention_kernel<T, NV><<<grid, kThreads, lds, stream>>>(a);
+  return PK_CHECK_LAUNCH();
+}
+
+template <typename T>
+int launch_pooled(const PooledArgs& a, dim3 grid, int VW, hipStream_t stream) {
+  const size_t lds = lds_bytes(a.D, VW, a.BK);
+  const int nv = (VW + 15) / 16;
+  if (nv <= 1) return launch_one<T, 1>(a, grid, lds, stream);
+  if (nv <= 2) return launch_one<T, 2>(a, grid, lds, stream);
+  if (nv <= 4) return launch_one<T, 4>(a, grid, lds, stream);
+  if (nv <= 8) return launch_one<T, 8>(a, grid, lds, stream);
+  if (nv <= 16) return launch_one<T, 16>(a, grid, lds, stream);
+  if (nv <= 32) return launch_one<T, 32>(a, grid, lds, stream);
+  return launch_one<T, 64>(a, grid, lds, stream);
+}
+
+// one wave per (token, head)
+template <typename OT>
+__global__ void __launch_bounds__(64)
+mix_heads_kernel(OT* __restrict__ out, int64_t out_stride, const float* __restrict__ o, const float* __restrict__ talk, int H,
+                 int VG, int V, float post) {
+  const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  OT* dst = out + static_cast<int64_t>(t) * out_stride + static_cast<int64_t>(h) * V;
+  const float* row = o + static_cast<int64_t>(t) * H * VG * V;
+  if (!talk) {
+    for (int c = lane; c < V; c += 64) st<OT>(dst + c, post * row[static_cast<int64_t>(h) * VG * V + c]);
+    return;
+  }
+  const int vh = h / (H / VG);
+  for (int c = lane; c < V; c += 64) {
+    float acc = 0.f;
+    for (int g = 0; g < H; ++g) acc += talk[h * H + g] * row[(static_cast<int64_t>(g) * VG + vh) * V + c];
+    st<OT>(dst + c, post * acc);
+  }
+}
+
+}  // namespace
+
+// caches [blocks, G, bs, D | V] of element type dt; a token at the last position of a block writes the block's means
+PK_EXPORT int pkm_pool_update(const void* k_cache, const void* v_cache, void* kp_cache, void* vp_cache,
+                              const void* positions, const void* token_seq, const void* block_tables, long long bt_stride,
+                              int T, int G, int D, int V, int bs, int pool, int dt, hipStream_t stream) {
+  if (T <= 0 || pool <= 0) return 0;
+  if (G < 1 || D < 1 || V < 1 || bs < 1) return -1;
+  const dim3 grid(T, G);
+  PKM_DISPATCH(dt, E, pool_update_kernel<E><<<grid, 256, 0, stream>>>(
+                          static_cast<const E*>(k_cache), static_cast<const E*>(v_cache), static_cast<E*>(kp_cache),
+                          static_cast<E*>(vp_cache), static_cast<const int*>(positions), static_cast<const int*>(token_seq),
+                          static_cast<const int*>(block_tables), bt_stride, G, D, V, bs, pool));
+  return PK_CHECK_LAUNCH();
+}
+
+// out fp32 [T, H, VG, V] (VG = G with all_values, else 1); q [T, H, D]; kp / vp null with pool = 0
+PK_EXPORT int pkm_pooled_attention(void* out, const void* q, const void* k_cache, const void* v_cache, const void* kp_cache,
+                                   const void* vp_cache, const void* block_tables, long long bt_stride, const void* cu_q,
+                                   const void* context_lens, const void* sink, int n_seqs, int T, int H, int G, int D, int V,
+                                   int bs, float scale, float softcap, int window, int pool, int all_values, int dt,
+                                   hipStream_t stream) {
+  if (T <= 0 || n_seqs <= 0) return 0;
+  if (H < 1 || G < 1 || H % G || D < 1 || V < 1 || bs < 1 || window < 0 || pool < 0) return -1;
+  if (pool > 0 && (!kp_cache || !vp_cache || window <= 0)) return -1;
+  const int VW = (all_values ? G : 1) * V;
+  if (VW > 1024) return -1;
+  PooledArgs a{static_cast<float*>(out), q, k_cache, v_cache, kp_cache, vp_cache, static_cast<const int*>(block_tables),
+               bt_stride, static_cast<const int*>(cu_q), static_cast<const int*>(context_lens),
+               static_cast<const float*>(sink), n_seqs, H, G, D, V, bs, key_tile(D, VW), scale, softcap, window, pool,
+               all_values};
+  if (a.BK == 0) return -1;
+  const int R = H / G;
+  // an upper bound of the row tiles: every sequence's rows rounded up
+  const int tiles = (T * R + kBQ - 1) / kBQ + n_seqs;
+  const dim3 grid(tiles, G);
+  if (dt == kBF16) return launch_pooled<bf16_t>(a, grid, VW, stream);
+  if (dt == kF32) return launch_pooled<float>(a, grid, VW, stream);
+  return -2;
+}
+
+// o fp32 [T, H, VG, V]; talk [H, H] fp32 (VG = G) or null (VG = 1); out rows out_stride elements apart
+PK_EXPORT int pkm_mix_heads(void* out, long long out_stride, int out_dt, const void* o, const void* talk, int T, int H,
+                            int VG, int V, float post, hipStream_t stream) {
+  if (T <= 0) return 0;
+  if (H < 1 || VG < 1 || H % VG || V < 1 || (talk == nullptr && VG != 1)) return -1;
+  const dim3 grid(T, H);
+  PKM_DISPATCH(out_dt, O, mix_heads_kernel<O><<<grid, 64, 0, stream>>>(static_cast<O*>(out), out_stride,
+                                                                       static_cast<const float*>(o),
+                                                                       static_cast<const float*>(talk), H, VG, V, post));
+  return PK_CHECK_LAUNCH();
+}

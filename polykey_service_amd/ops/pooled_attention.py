@@ -135,7 +135,7 @@ def mix_heads(o: torch.Tensor, talk: Optional[torch.Tensor], post: float, dtype:
     T, H, VG, V = o.shape
     if out is None:
         out = torch.empty((T, H * V), dtype=dtype, device=o.device)
-    assert out.shape == (T, H * V) and (talk is None) == (VG == 1) or (talk is None and VG == 1)
+    assert out.shape == (T, H * V) and (talk is not None or VG == 1)
     if not o.is_cuda:
         if talk is None:
             out.copy_((post * o[:, :, 0]).reshape(T, H * V))

@@ -70,7 +70,7 @@ def embed_rows_f32(table: torch.Tensor, ids: torch.Tensor) -> torch.Tensor:
     out = torch.empty((T, W), dtype=torch.float32, device=table.device)
     assert table.is_contiguous() and ids.dtype == torch.int32
     native.call("pkm_spread_rows", out.data_ptr(), table.data_ptr(), ids.data_ptr(), T, 1, W, table.shape[0],
-                native.dt_code(table.dtype), native.stream_ptr())
+                native.dt_code(table.dtype), 1.0, native.stream_ptr())
     return out
 
 

@@ -227,3 +227,104 @@ def forward(cfg: dict, tensors: dict, tokens):
     x = norm_one_plus(sum(xs), t64["final.norm"], eps)
     return x @ t64["embed"].T, torch.stack(after)
 
+
+
+# ------------------------------------------------------------------ small configurations and random weights
+def make_config(pattern=("wkv:dense", "parallel:moe", "mamba1:moe", "parallel:none"), vocab=96, width=48, streams=2,
+                heads=4, kv_heads=2, dim=16, vdim=8, rot_dims=8, window=24, pool=5, conv=3, softcap=15.0, wheads=3,
+                wdim=12, inner=40, state=6, dt_rank=5, mconv=4, ff=56, experts=5, top=2, eff=24, shared=32, taps=3,
+                mult=0.5, scale=None):
+    """A config.json dict: ``pattern`` lists "mixer:feed-forward" per layer."""
+    layers = []
+    for item in pattern:
+        kind, ffk = item.split(":")
+        if kind == "wkv":
+            mixer = {"heads": wheads, "dim": wdim}
+        elif kind == "mamba1":
+            mixer = {"inner": inner, "state": state, "dt_rank": dt_rank, "conv": mconv}
+        else:
+            left = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "conv": conv, "scale": dim ** -0.5,
+                    "softcap": softcap, "mask": {"size": window, "pool": pool}}
+            if rot_dims:
+                left["rot"] = {"dims": rot_dims, "base": 1000.0}
+            mixer = {"left": left, "right": {"heads": wheads, "dim": wdim}, "left_scale": 0.7, "right_scale": 1.2}
+        mlp = None
+        if ffk == "dense":
+            mlp = {"kind": "dense", "ff": ff, "limit": 1.5}
+        elif ffk == "moe":
+            mlp = {"kind": "moe", "router": {"experts": experts, "top": top}, "expert": {"ff": eff}}
+            if shared:
+                mlp["shared"] = {"ff": shared}
+        layers.append({"type": kind, "mixer": mixer, "mlp": mlp})
+    cfg = {"architecture": "Bibezen", "vocab": vocab, "width": width, "norm": {"eps": 1e-5}, "residual_mult": mult,
+           "embedding": {"scale": scale if scale is not None else float(width) ** 0.5}, "layers": layers}
+    if streams:
+        cfg["streams"] = streams
+    if taps:
+        cfg["canon"] = {"taps": taps}
+    return cfg
+
+
+def random_model(cfg, seed=0, std=None):
+    """Random bf16-representable tensors under the checkpoint names."""
+    g = torch.Generator().manual_seed(seed)
+    W, S = cfg["width"], cfg.get("streams", 0)
+    out = {}
+
+    def r(name, shape, s, mean=0.0):
+        out[name] = (mean + torch.randn(shape, generator=g) * s).to(torch.bfloat16).float()
+    fan = lambda n: std if std is not None else n ** -0.5
+
+    def wkv_weights(p, m):
+        n = m["heads"] * m["dim"]
+        for x in "rkvgw":
+            r(p + "mu." + x, (W,), 0.25, 0.5)
+        for x in "rkvg":
+            r(p + x, (n, W), fan(W))
+        r(p + "w1", (7, W), fan(W)), r(p + "w2", (n, 7), 0.4), r(p + "w0", (n,), 1.5, -1.0)
+        r(p + "u", (m["heads"], m["dim"]), 0.5), r(p + "norm", (n,), 0.1, 1.0), r(p + "o", (W, n), fan(n))
+
+    r("embed", (cfg["vocab"], W), W ** -0.5), r("final.norm", (W,), 0.1)
+    for i, l in enumerate(cfg["layers"]):
+        p, m = f"l{i}.", l["mixer"]
+        for q in ["1"] + (["2"] if l["mlp"] is not None else []):
+            r(p + "norm" + q, (W,), 0.1)
+            if S:
+                r(p + f"hc{q}.in", (S,), 0.15, 1.0 / S), r(p + f"hc{q}.out", (S,), 0.2, 1.0)
+                r(p + f"hc{q}.mix", (S, S), 0.1)
+                out[p + f"hc{q}.mix"] = (out[p + f"hc{q}.mix"] + torch.eye(S)).to(torch.bfloat16).float()
+        if (cfg.get("canon") or {}).get("taps"):
+            r(p + "canon1", (W, cfg["canon"]["taps"]), 0.25)
+        if l["type"] == "wkv":
+            wkv_weights(p + "mix.", m)
+        elif l["type"] == "mamba1":
+            I, N, R, K = m["inner"], m["state"], m["dt_rank"], m["conv"]
+            r(p + "mix.in", (2 * I, W), fan(W)), r(p + "mix.conv", (I, K), 0.4), r(p + "mix.conv.b", (I,), 0.1)
+            r(p + "mix.x", (R + 2 * N, I), fan(I)), r(p + "mix.dt", (I, R), fan(R)), r(p + "mix.dt.b", (I,), 1.0, -1.5)
+            r(p + "mix.A_log", (I, N), 0.5, 0.3), r(p + "mix.D", (I,), 0.5), r(p + "mix.o", (W, I), fan(I))
+        else:
+            a, q = m["left"], p + "mix.left."
+            H, G, D, V = a["heads"], a["kv_heads"], a["dim"], a["vdim"]
+            for n, rows in (("q", H * D), ("k", G * D), ("v", G * V)):
+                r(q + n, (rows, W), fan(W)), r(q + n + ".b", (rows,), 0.1)
+                if a.get("conv"):
+                    r(q + n + ".conv", (rows, a["conv"]), 0.5)
+            r(q + "q.norm", (D,), 0.1, 1.0), r(q + "k.norm", (D,), 0.1, 1.0), r(q + "sink", (H,), 1.0)
+            r(q + "talk", (H, H), 0.2)
+            out[q + "talk"] = (out[q + "talk"] + torch.eye(H)).to(torch.bfloat16).float()
+            r(q + "o", (W, H * V), fan(H * V))
+            wkv_weights(p + "mix.right.", m["right"])
+        f = l["mlp"]
+        if f is None:
+            continue
+        if f["kind"] == "dense":
+            r(p + "mlp.gate", (f["ff"], W), fan(W)), r(p + "mlp.up", (f["ff"], W), fan(W)), r(p + "mlp.down", (W, f["ff"]), fan(f["ff"]))
+        else:
+            r(p + "mlp.router", (f["router"]["experts"], W), 0.6)
+            names = [(f"e{e}", f["expert"]["ff"]) for e in range(f["router"]["experts"])]
+            if f.get("shared"):
+                names.append(("shared", f["shared"]["ff"]))
+            for n, ffn in names:
+                r(p + f"mlp.{n}.gate", (ffn, W), fan(W)), r(p + f"mlp.{n}.up", (ffn, W), fan(W))
+                r(p + f"mlp.{n}.down", (W, ffn), fan(ffn))
+    return out
