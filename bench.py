@@ -105,9 +105,9 @@ def parse_args(argv=None):
                          "sizes, e.g. '2k,4k' (presets <family>-<size>; random weights, one GPU, no RPC)")
     ap.add_argument("--compare-family", default="sapapel",
                     help="--compare-families: the family measured beside the --compare-with family (sapapel, kivezen, "
-                         "nopunex)")
+                         "nopunex, bibezen)")
     ap.add_argument("--compare-with", default="mixtral",
-                    help="--compare-families: the family measured beside it at equal layer sizes (mixtral; kivezen for nopunex)")
+                    help="--compare-families: the family measured beside it at equal layer sizes (mixtral; kivezen for nopunex and bibezen)")
     ap.add_argument("--compare-batch", type=int, default=32, help="--compare-families: sequences")
     ap.add_argument("--compare-prompt", type=int, default=1024, help="--compare-families: prompt tokens per sequence")
     ap.add_argument("--compare-decode", type=int, default=128, help="--compare-families: decoded tokens per sequence")

@@ -57,9 +57,48 @@ def rotate_halves(x, dims, base):
     return out
 
 
+def pooled_softmax(q, k, v, scale, cap=0.0, size=0, P=0, sink=None, talk=None):
+    """q [T, H, D], k [T, G, D], v [T, G, V] of one sequence from position 0.  Query i sees keys
+    max(0, i - size + 1) .. i (size 0: all) and the mean key / value of every block b of P positions with
+    b P + P - 1 <= i - size; s = cap tanh(q . k scale / cap); the denominator also holds exp(sink_h);
+    the weights of all heads are mixed by talk [H, H] before they meet head h's own values.  -> [T, H, V]"""
+    T, H, D = q.shape
+    G, V = k.shape[1], v.shape[2]
+    nb = T // P if (P and size) else 0
+    if nb:
+        kb, vb = k[:nb * P].view(nb, P, G, D).mean(1), v[:nb * P].view(nb, P, G, V).mean(1)
+    rep = H // G
+    wts = torch.zeros((H, T, T + nb), dtype=D64)      # softmax weights over single keys then blocks
+    for i in range(T):
+        seen = torch.zeros(T + nb, dtype=torch.bool)
+        seen[(max(0, i - size + 1) if size else 0):i + 1] = True
+        for b in range(nb):
+            if b * P + P - 1 <= i - size:
+                seen[T + b] = True
+        for hh in range(H):
+            g = hh // rep
+            sc = torch.cat([k[:, g] @ q[i, hh], kb[:, g] @ q[i, hh]] if nb else [k[:, g] @ q[i, hh]]) * scale
+            if cap:
+                sc = cap * torch.tanh(sc / cap)
+            sc = sc[seen]
+            m = sc.max()
+            if sink is not None:
+                m = torch.maximum(m, sink[hh])
+            e = torch.exp(sc - m)
+            den = e.sum() + (torch.exp(sink[hh] - m) if sink is not None else 0.0)
+            wts[hh, i, seen] = e / den
+    if talk is not None:
+        wts = torch.einsum("hg,gij->hij", talk, wts)
+    o = torch.zeros((T, H, V), dtype=D64)
+    for hh in range(H):
+        g = hh // rep
+        o[:, hh] = wts[hh] @ (torch.cat([v[:, g], vb[:, g]], 0) if nb else v[:, g])
+    return o
+
+
 def pooled_window_attention(h, t, s, eps):
-    """The softmax attention branch: biased projections, filters, head norms, rotation, capped scores,
-    a window of single keys plus block means behind it, a sink in the denominator, head mixing."""
+    """The softmax attention branch: biased projections, filters, weighted unit RMS per head,
+    rotation, then :func:`pooled_softmax` and the output projection."""
     T = h.shape[0]
     H, G, D, V = s["heads"], s["kv_heads"], s["dim"], s["vdim"]
 
@@ -79,41 +118,8 @@ def pooled_window_attention(h, t, s, eps):
     if rot:
         q, k = rotate_halves(q, rot["dims"], rot["base"]), rotate_halves(k, rot["dims"], rot["base"])
     mask = s.get("mask") or {}
-    size, P = mask.get("size", 0), mask.get("pool", 0)
-    cap = s.get("softcap", 0.0)
-    nb = T // P if P else 0
-    if nb:
-        kb, vb = k[:nb * P].view(nb, P, G, D).mean(1), v[:nb * P].view(nb, P, G, V).mean(1)
-    rep = H // G
-    wts = torch.zeros((H, T, T + nb), dtype=D64)      # softmax weights over single keys then blocks
-    for i in range(T):
-        seen = torch.zeros(T + nb, dtype=torch.bool)
-        lo = max(0, i - size + 1) if size else 0
-        seen[lo:i + 1] = True
-        if size:
-            for b in range(nb):
-                if b * P + P - 1 <= i - size:
-                    seen[T + b] = True
-        for hh in range(H):
-            g = hh // rep
-            sc = torch.cat([k[:, g] @ q[i, hh], kb[:, g] @ q[i, hh]] if nb else [k[:, g] @ q[i, hh]]) * s["scale"]
-            if cap:
-                sc = cap * torch.tanh(sc / cap)
-            sc = sc[seen]
-            m = sc.max()
-            sink = t["sink"][hh] if "sink" in t else None
-            if sink is not None:
-                m = torch.maximum(m, sink)
-            e = torch.exp(sc - m)
-            den = e.sum() + (torch.exp(sink - m) if sink is not None else 0.0)
-            wts[hh, i, seen] = e / den
-    if "talk" in t:
-        wts = torch.einsum("hg,gij->hij", t["talk"], wts)
-    o = torch.zeros((T, H, V), dtype=D64)
-    for hh in range(H):
-        g = hh // rep
-        vals = torch.cat([v[:, g], vb[:, g]], 0) if nb else v[:, g]
-        o[:, hh] = wts[hh] @ vals
+    o = pooled_softmax(q, k, v, s["scale"], s.get("softcap", 0.0), mask.get("size", 0), mask.get("pool", 0),
+                       t.get("sink"), t.get("talk"))
     return o.reshape(T, H * V) @ t["o"].T
 
 
