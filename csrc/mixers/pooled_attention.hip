@@ -28,11 +28,12 @@ namespace {
 template <typename T>
 __global__ void __launch_bounds__(256)
 pool_update_kernel(const T* __restrict__ k_cache, const T* __restrict__ v_cache, T* __restrict__ kp_cache,
-                   T* __restrict__ vp_cache, const int* __restrict__ positions, const int* __restrict__ token_seq,
-                   const int* __restrict__ block_tables, int64_t bt_stride, int G, int D, int V, int bs, int pool) {
+                   T* __restrict__ vp_cache, const int* __restrict__ positions, const int* __restrict__ slot_mapping,
+                   const int* __restrict__ token_seq, const int* __restrict__ block_tables, int64_t bt_stride, int G, int D,
+                   int V, int bs, int pool) {
   const int t = blockIdx.x, g = blockIdx.y;
   const int pos = positions[t];
-  if (pos < 0 || (pos + 1) % pool != 0) return;
+  if (pos < 0 || (pos + 1) % pool != 0 || (slot_mapping && slot_mapping[t] < 0)) return;
   const int* bt = block_tables + static_cast<int64_t>(token_seq[t]) * bt_stride;
   const int b = pos / pool;
   const int64_t dst = (static_cast<int64_t>(bt[b / bs]) * G + g) * bs + b % bs;
@@ -283,15 +284,18 @@ mix_heads_kernel(OT* __restrict__ out, int64_t out_stride, const float* __restri
 }  // namespace
 
 // caches [blocks, G, bs, D | V] of element type dt; a token at the last position of a block writes the block's means
+// (not a token whose slot_mapping entry is negative: it caches nothing)
 PK_EXPORT int pkm_pool_update(const void* k_cache, const void* v_cache, void* kp_cache, void* vp_cache,
-                              const void* positions, const void* token_seq, const void* block_tables, long long bt_stride,
+                              const void* positions, const void* slot_mapping, const void* token_seq,
+                              const void* block_tables, long long bt_stride,
                               int T, int G, int D, int V, int bs, int pool, int dt, hipStream_t stream) {
   if (T <= 0 || pool <= 0) return 0;
   if (G < 1 || D < 1 || V < 1 || bs < 1) return -1;
   const dim3 grid(T, G);
   PKM_DISPATCH(dt, E, pool_update_kernel<E><<<grid, 256, 0, stream>>>(
                           static_cast<const E*>(k_cache), static_cast<const E*>(v_cache), static_cast<E*>(kp_cache),
-                          static_cast<E*>(vp_cache), static_cast<const int*>(positions), static_cast<const int*>(token_seq),
+                          static_cast<E*>(vp_cache), static_cast<const int*>(positions),
+                          static_cast<const int*>(slot_mapping), static_cast<const int*>(token_seq),
                           static_cast<const int*>(block_tables), bt_stride, G, D, V, bs, pool));
   return PK_CHECK_LAUNCH();
 }

@@ -219,7 +219,8 @@ class ParallelMixer(nn.Module):
                                 q_norm=self.q_norm, k_norm=self.k_norm, eps=eps)
         pooled = s.window > 0 and s.pool > 0
         if pooled:
-            pa_ops.pool_update(kc, vc, cache["kp"], cache["vp"], positions, md.token_seq, md.block_tables, s.pool)
+            pa_ops.pool_update(kc, vc, cache["kp"], cache["vp"], positions, md.token_seq, md.block_tables, s.pool,
+                               md.slot_mapping)
         o = pa_ops.pooled_attention(q, kc, vc, cache.get("kp"), cache.get("vp"), md.block_tables, md.cu_q, md.context_lens,
                                     md.num_seqs, s.scale, s.softcap, s.window, s.pool if pooled else 0, self.sink,
                                     all_values=self.talk is not None)

@@ -30,10 +30,12 @@ def _rows(cache: torch.Tensor, bt: torch.Tensor, idx: torch.Tensor) -> torch.Ten
 
 
 def pool_update(k_cache: torch.Tensor, v_cache: torch.Tensor, kp_cache: torch.Tensor, vp_cache: torch.Tensor,
-                positions: torch.Tensor, token_seq: torch.Tensor, block_tables: torch.Tensor, pool: int) -> None:
+                positions: torch.Tensor, token_seq: torch.Tensor, block_tables: torch.Tensor, pool: int,
+                slot_mapping: Optional[torch.Tensor] = None) -> None:
     """For every token of the step at the last position of a block of ``pool``: the mean of the
     block's rows of k_cache / v_cache goes to entry position // pool of kp_cache / vp_cache (after
-    the step's rows are in the caches).  Caches are [blocks, heads, block_size, width]."""
+    the step's rows are in the caches).  Caches are [blocks, heads, block_size, width].  Tokens whose
+    ``slot_mapping`` entry is negative cache nothing (padded rows of a decode graph) and are skipped."""
     T = positions.numel()
     if pool <= 0 or T == 0:
         return
@@ -41,7 +43,7 @@ def pool_update(k_cache: torch.Tensor, v_cache: torch.Tensor, kp_cache: torch.Te
     if not k_cache.is_cuda:
         for t in range(T):
             p = int(positions[t])
-            if (p + 1) % pool:
+            if (p + 1) % pool or (slot_mapping is not None and int(slot_mapping[t]) < 0):
                 continue
             bt = block_tables[int(token_seq[t])]
             idx = torch.arange(p - pool + 1, p + 1)
@@ -52,7 +54,8 @@ def pool_update(k_cache: torch.Tensor, v_cache: torch.Tensor, kp_cache: torch.Te
         return
     assert k_cache.shape == kp_cache.shape and v_cache.shape == vp_cache.shape and block_tables.stride(1) == 1
     native.call("pkm_pool_update", k_cache.data_ptr(), v_cache.data_ptr(), kp_cache.data_ptr(), vp_cache.data_ptr(),
-                positions.data_ptr(), token_seq.data_ptr(), block_tables.data_ptr(), block_tables.stride(0), T,
+                positions.data_ptr(), native.ptr(slot_mapping), token_seq.data_ptr(), block_tables.data_ptr(),
+                block_tables.stride(0), T,
                 k_cache.shape[1], k_cache.shape[3], v_cache.shape[3], bs, int(pool), native.dt_code(k_cache.dtype),
                 native.stream_ptr())
 
