@@ -9,7 +9,7 @@ are fp32):
 
     h   = N1(sum_s in1[s] xs[s]) -> a ;  h <- h + filter(h)                   HIP  hyper.hip, short_conv.hip
     wkv:       mixes of h with the previous token's h, one per projection      HIP  wkv.hip
-               r, k, v, g = mix_n @ W_n^T ; z = tanh(mix_w @ W1^T) @ W2^T      batched / library GEMMs
+               r, k, v, g = mix_n @ W_n^T ; z = tanh(mix_w @ W1^T) @ W2^T      hipBLASLt / decode GEMM
                o = (S + diag(u) k v^T)^T r ; S <- diag(exp(-exp(z + w0))) S + k v^T   (state [H, D, D] fp32 per slot)
                o = unit_rms_per_head(o) * w * silu(g)                          HIP  head_norm_gate
     mamba1:    x | z = h @ Win^T ; x = silu(filter(x) + b) ; dt | B | C = x @ Wx^T ; d = dt @ Wdt^T
@@ -58,6 +58,17 @@ def _f32(t: torch.Tensor, device) -> nn.Parameter:
     return _p(t.to(device=device, dtype=torch.float32))
 
 
+def _project_into(x: torch.Tensor, w: torch.Tensor, packed: Optional[torch.Tensor], out: torch.Tensor) -> torch.Tensor:
+    """x @ w^T written to ``out`` (a plane of a larger buffer): decode-sized rows on the
+    weight-streaming GEMM (split-K slabs summed into ``out``), else the library GEMM."""
+    if gemm.skinny_ok(x, w):
+        S = gemm.choose_split(w.shape[0], x.shape[1], x.shape[0])
+        if S > 1:
+            ws = torch.empty(S * x.shape[0] * w.shape[0], dtype=torch.float32, device=x.device)
+            return gemm.reduce_partial(gemm.linear_partial(x, w, ws, S, packed=packed), out)
+    return gemm.linear(x, w, out=out, packed=packed)
+
+
 class WkvMixer(nn.Module):
     """Weights of one wkv time-mixing branch.  ``activation`` leaves the normed, gated head outputs
     (times ``post``) for the output projection of whoever owns the branch."""
@@ -66,13 +77,15 @@ class WkvMixer(nn.Module):
         super().__init__()
         self.spec, self.width = spec, width
         self.mu = None       # [5, W] fp32: r, k, v, g, w
-        self.w_in = None     # [4, H*D, W]: r, k, v, g
+        self.w_in = None     # r, k, v, g: four [H*D, W]
+        self.w_in_p = [None] * 4
         self.w1 = self.w2 = None    # [R, W], [H*D, R]
         self.w0 = self.u = self.norm_w = None   # [H*D] fp32
         self.w_o = self.w_o_p = None            # [W, H*D]
 
     def pack(self) -> None:
         self.w_o_p = _packed(self.w_o) if self.w_o is not None else None
+        self.w_in_p = [_packed(w) for w in self.w_in]
 
     def set(self, get, dtype, device, own_output: bool = True) -> None:
         s, W = self.spec, self.width
@@ -80,7 +93,7 @@ class WkvMixer(nn.Module):
         ws = [get(x) for x in "rkvg"]
         assert all(w.shape == (n, W) for w in ws) and get("w1").shape[1] == W and get("w2").shape == (n, get("w1").shape[0])
         self.mu = _f32(torch.stack([get("mu." + x).reshape(W) for x in "rkvgw"]), device)
-        self.w_in = _p(torch.stack(ws).to(device=device, dtype=dtype))
+        self.w_in = nn.ParameterList([_p(w.to(device=device, dtype=dtype)) for w in ws])
         self.w1, self.w2 = _p(get("w1").to(device=device, dtype=dtype)), _p(get("w2").to(device=device, dtype=dtype))
         self.w0, self.u, self.norm_w = (_f32(get(x).reshape(n), device) for x in ("w0", "u", "norm"))
         if own_output:
@@ -91,7 +104,9 @@ class WkvMixer(nn.Module):
         s = self.spec
         T, n = h.shape[0], s.heads * s.dim
         mixes = wkv_ops.shift_mix(h, self.mu, cache["prev"], md.token_seq, md.cu_q, md.num_seqs, positions, md.state_slots)
-        rkvg = torch.bmm(mixes[:4], self.w_in.transpose(1, 2))                                  # [4, T, H*D]
+        rkvg = torch.empty((4, T, n), dtype=h.dtype, device=h.device)
+        for i in range(4):       # one projection per mix (a batched library GEMM returned NaN at 8192 x 2048 x 2048 bf16)
+            _project_into(mixes[i], self.w_in[i], self.w_in_p[i], rkvg[i])
         z = gemm.linear(wkv_ops.tanh_(gemm.linear(mixes[4], self.w1)), self.w2)
         o = wkv_ops.wkv_recurrence(rkvg, z, self.w0, self.u, cache["wkv"], md.cu_q, md.num_seqs, positions,
                                    md.state_slots, s.heads, s.dim)
