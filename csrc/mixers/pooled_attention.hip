@@ -64,7 +64,84 @@ struct PooledArgs {
   int n_seqs, H, G, D, V, bs, BK;
   float scale, softcap;
   int window, pool, all_values;
+  // few rows (decoded tokens): the key tiles are dealt to n_parts workgroups per row tile, which leave
+  // (max, sum, unnormalised sums) in the workspace for pooled_merge_kernel (the sink joins there)
+  int n_parts;
+  float* ws_acc;  // [T * H, n_parts, VW]
+  float* ws_ml;   // [T * H, n_parts, 2]
 };
+
+// 16 bytes of a cache row as floats
+template <typename T>
+struct Chunk;
+template <>
+struct Chunk<float> {
+  static constexpr int N = 4;
+  __device__ static __forceinline__ void load(const float* p, float* f) {
+    const float4 v = *reinterpret_cast<const float4*>(p);
+    f[0] = v.x, f[1] = v.y, f[2] = v.z, f[3] = v.w;
+  }
+};
+template <>
+struct Chunk<bf16_t> {
+  static constexpr int N = 8;
+  __device__ static __forceinline__ void load(const bf16_t* p, float* f) {
+    const uint4 v = *reinterpret_cast<const uint4*>(p);
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      f[2 * i] = __uint_as_float(w[i] << 16);
+      f[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+    }
+  }
+};
+
+// rows [j0, j0 + BK) x width columns of a paged cache into an LDS tile with row stride `stride`:
+// 16-byte loads when the width allows (all loads of a pass are issued before the first LDS store)
+template <typename T>
+__device__ __forceinline__ void stage_tile(float* tile, int stride, const T* cache, const int* bt, int bs, int heads,
+                                           int head0, int n_heads, int width, int k0, int nk, int BK, int tid) {
+  constexpr int N = Chunk<T>::N;
+  const int W = n_heads * width;  // columns of the tile: n_heads heads side by side
+  if (width % N == 0) {
+    const int per = W / N, units = BK * per;
+    constexpr int kPass = 4;
+    for (int u0 = 0; u0 < units; u0 += kPass * kThreads) {
+      float f[kPass][N];
+#pragma unroll
+      for (int p = 0; p < kPass; ++p) {
+        const int u = u0 + p * kThreads + tid;
+        const int j = u / per, c = (u - j * per) * N;
+        if (u < units && j < nk) {
+          const int key = k0 + j, g = c / width, cc = c - g * width;
+          Chunk<T>::load(cache + ((static_cast<int64_t>(bt[key / bs]) * heads + head0 + g) * bs + key % bs) * width + cc, f[p]);
+        } else {
+#pragma unroll
+          for (int i = 0; i < N; ++i) f[p][i] = 0.f;
+        }
+      }
+#pragma unroll
+      for (int p = 0; p < kPass; ++p) {
+        const int u = u0 + p * kThreads + tid;
+        if (u < units) {
+          const int j = u / per, c = (u - j * per) * N;
+#pragma unroll
+          for (int i = 0; i < N; ++i) tile[j * stride + c + i] = f[p][i];
+        }
+      }
+    }
+    return;
+  }
+  for (int e = tid; e < BK * W; e += kThreads) {
+    const int j = e / W, c = e - j * W;
+    float v = 0.f;
+    if (j < nk) {
+      const int key = k0 + j, g = c / width, cc = c - g * width;
+      v = ld<T>(cache + ((static_cast<int64_t>(bt[key / bs]) * heads + head0 + g) * bs + key % bs) * width + cc);
+    }
+    tile[j * stride + c] = v;
+  }
+}
 
 __device__ __forceinline__ int blocks_seen(int pos, int window, int pool) {
   if (window <= 0 || pool <= 0) return 0;
@@ -123,8 +200,9 @@ __global__ void __launch_bounds__(kThreads) pooled_attention_kernel(PooledArgs a
   if (tid < kBQ) {
     const int row = row0 + tid;
     const int h = kh * R + (row < n_rows ? row % R : 0);
-    m_s[tid] = a.sink ? a.sink[h] : -INFINITY;  // the sink is a key without a value
-    l_s[tid] = a.sink ? 1.f : 0.f;
+    const bool sink_here = a.sink && a.n_parts <= 1;
+    m_s[tid] = sink_here ? a.sink[h] : -INFINITY;  // the sink is a key without a value
+    l_s[tid] = sink_here ? 1.f : 0.f;
   }
   const int first_pos = ctx - qlen + row0 / R;
   const int last_pos = ctx - qlen + (min(row0 + kBQ, n_rows) - 1) / R;
@@ -134,6 +212,7 @@ __global__ void __launch_bounds__(kThreads) pooled_attention_kernel(PooledArgs a
   __syncthreads();
 
   // part 0: the block means (entries [0, blocks seen by the tile's last row)); part 1: single keys
+  int tile_no = 0;
   for (int part = 0; part < 2; ++part) {
     const T* kc = static_cast<const T*>(part ? a.k_cache : a.kp_cache);
     const T* vc = static_cast<const T*>(part ? a.v_cache : a.vp_cache);
@@ -146,26 +225,10 @@ __global__ void __launch_bounds__(kThreads) pooled_attention_kernel(PooledArgs a
       k_begin = (first_pos >= 0 && a.window > 0) ? max(0, first_pos - a.window + 1) / BK * BK : 0;
     }
     for (int k0 = k_begin; k0 < k_end; k0 += BK) {
+      if (a.n_parts > 1 && (tile_no++) % a.n_parts != static_cast<int>(blockIdx.z)) continue;
       const int nk = min(BK, k_end - k0);
-      for (int e = tid; e < BK * D; e += kThreads) {
-        const int j = e / D, c = e - j * D;
-        float v = 0.f;
-        if (j < nk) {
-          const int key = k0 + j;
-          v = ld<T>(kc + ((static_cast<int64_t>(bt[key / bs]) * G + kh) * bs + key % bs) * D + c);
-        }
-        ks[j * DS + c] = v;
-      }
-      for (int e = tid; e < BK * VW; e += kThreads) {
-        const int j = e / VW, c = e - j * VW;
-        float v = 0.f;
-        if (j < nk) {
-          const int key = k0 + j;
-          const int g = a.all_values ? c / V : kh, cc = a.all_values ? c - g * V : c;
-          v = ld<T>(vc + ((static_cast<int64_t>(bt[key / bs]) * G + g) * bs + key % bs) * V + cc);
-        }
-        vs[j * VS + c] = v;
-      }
+      stage_tile<T>(ks, DS, kc, bt, bs, G, kh, 1, D, k0, nk, BK, tid);
+      stage_tile<T>(vs, VS, vc, bt, bs, G, a.all_values ? 0 : kh, VG, V, k0, nk, BK, tid);
       __syncthreads();
       float tmax = -INFINITY;
       for (int j = kg; j < BK; j += 16) {
@@ -215,11 +278,46 @@ __global__ void __launch_bounds__(kThreads) pooled_attention_kernel(PooledArgs a
   const float l = l_s[qi];
   const float inv = l > 0.f ? 1.f / l : 0.f;
   if (!live) return;
+  if (a.n_parts > 1) {
+    const int64_t slot = (static_cast<int64_t>(q0 + my_tl) * H + my_h) * a.n_parts + blockIdx.z;
+    float* dst = a.ws_acc + slot * VW;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int c = kg + 16 * i;
+      if (c < VW) dst[c] = acc[i];
+    }
+    if (kg == 0) {
+      a.ws_ml[2 * slot] = m_s[qi];
+      a.ws_ml[2 * slot + 1] = l;
+    }
+    return;
+  }
   float* dst = a.out + (static_cast<int64_t>(q0 + my_tl) * H + my_h) * VW;
 #pragma unroll
   for (int i = 0; i < NV; ++i) {
     const int c = kg + 16 * i;
     if (c < VW) dst[c] = acc[i] * inv;
+  }
+}
+
+// out[t, h] from the parts' (max, sum, unnormalised sums) and the head's sink: one wave per (token, head)
+__global__ void __launch_bounds__(64)
+pooled_merge_kernel(float* __restrict__ out, const float* __restrict__ ws_acc, const float* __restrict__ ws_ml,
+                    const float* __restrict__ sink, int H, int VW, int n_parts) {
+  const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const int64_t row = static_cast<int64_t>(t) * H + h;
+  const float* ml = ws_ml + row * n_parts * 2;
+  float m = sink ? sink[h] : -INFINITY;
+  for (int p = 0; p < n_parts; ++p) m = fmaxf(m, ml[2 * p]);
+  float l = (sink && m != -INFINITY) ? expf(sink[h] - m) : 0.f;
+  for (int p = 0; p < n_parts; ++p)
+    if (ml[2 * p] != -INFINITY) l += ml[2 * p + 1] * expf(ml[2 * p] - m);
+  const float inv = l > 0.f ? 1.f / l : 0.f;
+  for (int c = lane; c < VW; c += 64) {
+    float acc = 0.f;
+    for (int p = 0; p < n_parts; ++p)
+      if (ml[2 * p] != -INFINITY) acc += ws_acc[(row * n_parts + p) * VW + c] * expf(ml[2 * p] - m);
+    out[row * VW + c] = acc * inv;
   }
 }
 
@@ -300,12 +398,13 @@ PK_EXPORT int pkm_pool_update(const void* k_cache, const void* v_cache, void* kp
   return PK_CHECK_LAUNCH();
 }
 
-// out fp32 [T, H, VG, V] (VG = G with all_values, else 1); q [T, H, D]; kp / vp null with pool = 0
+// out fp32 [T, H, VG, V] (VG = G with all_values, else 1); q [T, H, D]; kp / vp null with pool = 0; n_parts > 1:
+// workspaces ws_acc [T * H, n_parts, VG * V] and ws_ml [T * H, n_parts, 2] fp32
 PK_EXPORT int pkm_pooled_attention(void* out, const void* q, const void* k_cache, const void* v_cache, const void* kp_cache,
                                    const void* vp_cache, const void* block_tables, long long bt_stride, const void* cu_q,
                                    const void* context_lens, const void* sink, int n_seqs, int T, int H, int G, int D, int V,
-                                   int bs, float scale, float softcap, int window, int pool, int all_values, int dt,
-                                   hipStream_t stream) {
+                                   int bs, float scale, float softcap, int window, int pool, int all_values, int n_parts,
+                                   void* ws_acc, void* ws_ml, int dt, hipStream_t stream) {
   if (T <= 0 || n_seqs <= 0) return 0;
   if (H < 1 || G < 1 || H % G || D < 1 || V < 1 || bs < 1 || window < 0 || pool < 0) return -1;
   if (pool > 0 && (!kp_cache || !vp_cache || window <= 0)) return -1;
@@ -314,15 +413,18 @@ PK_EXPORT int pkm_pooled_attention(void* out, const void* q, const void* k_cache
   PooledArgs a{static_cast<float*>(out), q, k_cache, v_cache, kp_cache, vp_cache, static_cast<const int*>(block_tables),
                bt_stride, static_cast<const int*>(cu_q), static_cast<const int*>(context_lens),
                static_cast<const float*>(sink), n_seqs, H, G, D, V, bs, key_tile(D, VW), scale, softcap, window, pool,
-               all_values};
-  if (a.BK == 0) return -1;
+               all_values, n_parts, static_cast<float*>(ws_acc), static_cast<float*>(ws_ml)};
+  if (a.BK == 0 || n_parts < 1 || n_parts > 64 || (n_parts > 1 && (!ws_acc || !ws_ml))) return -1;
   const int R = H / G;
   // an upper bound of the row tiles: every sequence's rows rounded up
   const int tiles = (T * R + kBQ - 1) / kBQ + n_seqs;
-  const dim3 grid(tiles, G);
-  if (dt == kBF16) return launch_pooled<bf16_t>(a, grid, VW, stream);
-  if (dt == kF32) return launch_pooled<float>(a, grid, VW, stream);
-  return -2;
+  const dim3 grid(tiles, G, n_parts);
+  int rc = -2;
+  if (dt == kBF16) rc = launch_pooled<bf16_t>(a, grid, VW, stream);
+  if (dt == kF32) rc = launch_pooled<float>(a, grid, VW, stream);
+  if (rc != 0 || n_parts == 1) return rc;
+  pooled_merge_kernel<<<dim3(T, H), 64, 0, stream>>>(a.out, a.ws_acc, a.ws_ml, a.sink, H, VW, n_parts);
+  return PK_CHECK_LAUNCH();
 }
 
 // o fp32 [T, H, VG, V]; talk [H, H] fp32 (VG = G) or null (VG = 1); out rows out_stride elements apart

@@ -123,7 +123,7 @@ MIXER_SIGNATURES = {
     "pkm_selective_scan": [P, P, I64, P, I64, P, P, P, I64, P, P, I64, P, P, P, P, I32, I32, I32, I32, I32, P],
     "pkm_pool_update": [P, P, P, P, P, P, P, P, I64, I32, I32, I32, I32, I32, I32, I32, P],
     "pkm_pooled_attention": [P, P, P, P, P, P, P, I64, P, P, P, I32, I32, I32, I32, I32, I32, I32, F32, F32, I32, I32, I32,
-                             I32, P],
+                             I32, P, P, I32, P],
     "pkm_mix_heads": [P, I64, I32, P, P, I32, I32, I32, I32, F32, P],
 }
 _mixers: Optional[ctypes.CDLL] = None

@@ -122,11 +122,19 @@ def pooled_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
     assert q.is_contiguous() and q.dtype == k_cache.dtype == v_cache.dtype and k_cache.is_contiguous() and v_cache.is_contiguous()
     assert block_tables.stride(1) == 1 and (sink is None or (sink.dtype == torch.float32 and sink.numel() == H))
     assert pool == 0 or (kp_cache.shape == k_cache.shape and vp_cache.shape == v_cache.shape)
+    # few row tiles (decoded tokens): the key tiles of a row tile are dealt to several workgroups and merged
+    tiles = (-(-T * rep // 16) + n_seqs) * G
+    span = block_tables.shape[1] * bs if window <= 0 else min(block_tables.shape[1] * bs, window + 64)
+    n_parts = max(1, min(16, 1024 // tiles, span // 64))
+    ws_acc = ws_ml = None
+    if n_parts > 1:
+        ws_acc = torch.empty((T * H, n_parts, VG * V), dtype=torch.float32, device=q.device)
+        ws_ml = torch.empty((T * H, n_parts, 2), dtype=torch.float32, device=q.device)
     native.call("pkm_pooled_attention", out.data_ptr(), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
                 native.ptr(kp_cache) if pool else None, native.ptr(vp_cache) if pool else None, block_tables.data_ptr(),
                 block_tables.stride(0), cu_q.data_ptr(), context_lens.data_ptr(), native.ptr(sink), n_seqs, T, H, G, D, V,
-                bs, float(scale), float(softcap), int(window), int(pool), int(all_values), native.dt_code(q.dtype),
-                native.stream_ptr())
+                bs, float(scale), float(softcap), int(window), int(pool), int(all_values), n_parts, native.ptr(ws_acc),
+                native.ptr(ws_ml), native.dt_code(q.dtype), native.stream_ptr())
     return out
 
 
