@@ -149,7 +149,7 @@ __device__ __forceinline__ int blocks_seen(int pos, int window, int pool) {
   return n >= pool ? n / pool : 0;
 }
 
-// NV: output accumulators per thread = ceil(value columns / 16)
+// NV: output accumulators per thread and row = ceil(value columns / 64)
 template <typename T, int NV>
 __global__ void __launch_bounds__(kThreads) pooled_attention_kernel(PooledArgs a) {
   extern __shared__ float smem[];
@@ -176,6 +176,7 @@ __global__ void __launch_bounds__(kThreads) pooled_attention_kernel(PooledArgs a
   float* ps = vs + BK * VS;     // [kBQ][BK]
   float* m_s = ps + kBQ * BK;   // [kBQ] running max
   float* l_s = m_s + kBQ;       // [kBQ] running sum
+  float* r_s = l_s + kBQ;       // [kBQ] the current tile's rescale of each row's sums
   const int tid = threadIdx.x;
   const int qi = tid >> 4, kg = tid & 15;
   const int* bt = a.block_tables + static_cast<int64_t>(s) * a.bt_stride;
@@ -206,9 +207,15 @@ __global__ void __launch_bounds__(kThreads) pooled_attention_kernel(PooledArgs a
   }
   const int first_pos = ctx - qlen + row0 / R;
   const int last_pos = ctx - qlen + (min(row0 + kBQ, n_rows) - 1) / R;
-  float acc[NV];
+  // value sums: thread (rg, cl) owns rows 4 rg .. 4 rg + 3 and columns cl + 64 i, so a value read from LDS
+  // meets four rows; row groups past the tile's rows (decoded tokens: R rows) sit the products out
+  const int rg = tid >> 6, cl = tid & 63;
+  const bool pv_live = row0 + 4 * rg < n_rows;
+  float acc[4][NV];
 #pragma unroll
-  for (int i = 0; i < NV; ++i) acc[i] = 0.f;
+  for (int r = 0; r < 4; ++r)
+#pragma unroll
+    for (int i = 0; i < NV; ++i) acc[r][i] = 0.f;
   __syncthreads();
 
   // part 0: the block means (entries [0, blocks seen by the tile's last row)); part 1: single keys
@@ -232,15 +239,17 @@ __global__ void __launch_bounds__(kThreads) pooled_attention_kernel(PooledArgs a
       __syncthreads();
       float tmax = -INFINITY;
       for (int j = kg; j < BK; j += 16) {
-        float d = 0.f;
-        const float* qr = qs + qi * DS;
-        const float* kr = ks + j * DS;
-        for (int c = 0; c < D; ++c) d += qr[c] * kr[c];
-        d *= a.scale;
-        if (a.softcap > 0.f) d = a.softcap * tanhf(d / a.softcap);
         const int key = k0 + j;
-        const bool seen = part == 0 ? key < my_blocks : (key <= my_pos && key >= my_lo);
-        d = (j < nk && seen) ? d : -INFINITY;
+        const bool seen = j < nk && live && (part == 0 ? key < my_blocks : (key <= my_pos && key >= my_lo));
+        float d = -INFINITY;
+        if (seen) {
+          d = 0.f;
+          const float* qr = qs + qi * DS;
+          const float* kr = ks + j * DS;
+          for (int c = 0; c < D; ++c) d += qr[c] * kr[c];
+          d *= a.scale;
+          if (a.softcap > 0.f) d = a.softcap * tanhf(d / a.softcap);
+        }
         ps[qi * BK + j] = d;
         tmax = fmaxf(tmax, d);
       }
@@ -258,45 +267,65 @@ __global__ void __launch_bounds__(kThreads) pooled_attention_kernel(PooledArgs a
 #pragma unroll
       for (int o = 8; o > 0; o >>= 1) tsum += __shfl_xor(tsum, o, 64);
       const float resc = (m_old == -INFINITY) ? 0.f : expf(m_old - m_new);
+      if (kg == 0) r_s[qi] = resc;
       __syncthreads();  // every lane of the row has read m_old and its own scores
       if (kg == 0) {
         m_s[qi] = m_new;
         l_s[qi] = l_s[qi] * resc + tsum;
       }
+      if (pv_live) {
 #pragma unroll
-      for (int i = 0; i < NV; ++i) acc[i] *= resc;
-      for (int j = 0; j < nk; ++j) {
-        const float p = ps[qi * BK + j];
-        const float* vr = vs + j * VS + kg;
+        for (int r = 0; r < 4; ++r) {
+          const float rs = r_s[4 * rg + r];
 #pragma unroll
-        for (int i = 0; i < NV; ++i)
-          if (kg + 16 * i < VW) acc[i] += p * vr[16 * i];
+          for (int i = 0; i < NV; ++i) acc[r][i] *= rs;
+        }
+        for (int j = 0; j < nk; ++j) {
+          float p[4];
+#pragma unroll
+          for (int r = 0; r < 4; ++r) p[r] = ps[(4 * rg + r) * BK + j];
+          const float* vr = vs + j * VS + cl;
+#pragma unroll
+          for (int i = 0; i < NV; ++i) {
+            if (cl + 64 * i < VW) {
+              const float v = vr[64 * i];
+#pragma unroll
+              for (int r = 0; r < 4; ++r) acc[r][i] += p[r] * v;
+            }
+          }
+        }
       }
       __syncthreads();
     }
   }
-  const float l = l_s[qi];
-  const float inv = l > 0.f ? 1.f / l : 0.f;
-  if (!live) return;
-  if (a.n_parts > 1) {
-    const int64_t slot = (static_cast<int64_t>(q0 + my_tl) * H + my_h) * a.n_parts + blockIdx.z;
-    float* dst = a.ws_acc + slot * VW;
+  if (!pv_live) return;
 #pragma unroll
-    for (int i = 0; i < NV; ++i) {
-      const int c = kg + 16 * i;
-      if (c < VW) dst[c] = acc[i];
-    }
-    if (kg == 0) {
-      a.ws_ml[2 * slot] = m_s[qi];
-      a.ws_ml[2 * slot + 1] = l;
-    }
-    return;
-  }
-  float* dst = a.out + (static_cast<int64_t>(q0 + my_tl) * H + my_h) * VW;
+  for (int r = 0; r < 4; ++r) {
+    const int row = row0 + 4 * rg + r;
+    if (row >= n_rows) break;
+    const int tl = row / R, h = kh * R + row - tl * R;
+    const float l = l_s[4 * rg + r];
+    if (a.n_parts > 1) {
+      const int64_t slot = (static_cast<int64_t>(q0 + tl) * H + h) * a.n_parts + blockIdx.z;
+      float* dst = a.ws_acc + slot * VW;
 #pragma unroll
-  for (int i = 0; i < NV; ++i) {
-    const int c = kg + 16 * i;
-    if (c < VW) dst[c] = acc[i] * inv;
+      for (int i = 0; i < NV; ++i) {
+        const int c = cl + 64 * i;
+        if (c < VW) dst[c] = acc[r][i];
+      }
+      if (cl == 0) {
+        a.ws_ml[2 * slot] = m_s[4 * rg + r];
+        a.ws_ml[2 * slot + 1] = l;
+      }
+    } else {
+      const float inv = l > 0.f ? 1.f / l : 0.f;
+      float* dst = a.out + (static_cast<int64_t>(q0 + tl) * H + h) * VW;
+#pragma unroll
+      for (int i = 0; i < NV; ++i) {
+        const int c = cl + 64 * i;
+        if (c < VW) dst[c] = acc[r][i] * inv;
+      }
+    }
   }
 }
 
@@ -322,7 +351,7 @@ pooled_merge_kernel(float* __restrict__ out, const float* __restrict__ ws_acc, c
 }
 
 size_t lds_bytes(int D, int VW, int bk) {
-  return (static_cast<size_t>(kBQ) * (D + 1) + static_cast<size_t>(bk) * (D + 1 + VW + 1) + kBQ * bk + 2 * kBQ) * 4;
+  return (static_cast<size_t>(kBQ) * (D + 1) + static_cast<size_t>(bk) * (D + 1 + VW + 1) + kBQ * bk + 3 * kBQ) * 4;
 }
 
 // key tile: the largest of 64 / 32 / 16 whose tiles fit 60 KiB of LDS, else the largest of 32 / 16 / 8
@@ -349,14 +378,12 @@ int launch_one(const PooledArgs& a, dim3 grid, size_t lds, hipStream_t stream) {
 template <typename T>
 int launch_pooled(const PooledArgs& a, dim3 grid, int VW, hipStream_t stream) {
   const size_t lds = lds_bytes(a.D, VW, a.BK);
-  const int nv = (VW + 15) / 16;
+  const int nv = (VW + 63) / 64;
   if (nv <= 1) return launch_one<T, 1>(a, grid, lds, stream);
   if (nv <= 2) return launch_one<T, 2>(a, grid, lds, stream);
   if (nv <= 4) return launch_one<T, 4>(a, grid, lds, stream);
   if (nv <= 8) return launch_one<T, 8>(a, grid, lds, stream);
-  if (nv <= 16) return launch_one<T, 16>(a, grid, lds, stream);
-  if (nv <= 32) return launch_one<T, 32>(a, grid, lds, stream);
-  return launch_one<T, 64>(a, grid, lds, stream);
+  return launch_one<T, 16>(a, grid, lds, stream);
 }
 
 // one wave per (token, head)

@@ -7,7 +7,7 @@
 //   wkv         per (sequence, head), state S [D, D] fp32 (key channel, value channel):
 //                 w_t = exp(-exp(z_t + w0));  o_t = (S + diag(u) k_t v_t^T)^T r_t;  S <- diag(w_t) S + k_t v_t^T
 //               A wave owns 64 value columns of a (sequence, head); every lane keeps its column of S in
-//               registers; r, k, w and u k of a round of tokens are staged in LDS (one 16-byte
+//               registers; r, k, w and u k of a round of 16 tokens are staged in LDS (one 16-byte
 //               broadcast read per key channel).  Tokens are walked in order with the same order of
 //               sums whether a token arrives in a portion or alone.
 #include "mix_common.h"
@@ -57,15 +57,18 @@ __global__ void __launch_bounds__(256) tanh_kernel(T* __restrict__ x, int64_t n)
   if (i < n) st<T>(x + i, tanhf(ld<T>(x + i)));
 }
 
-constexpr int kRound = 8;  // tokens staged per round
+constexpr int kRound = 16;  // tokens staged per round
 
 // ND: key channels kept per lane (>= D).  grid (column groups of 64, H, sequences), one wave each.
+// A round's loads (r, k, z of every key channel, the lane's v of every token) are issued together
+// before their first use, so the wave waits for memory once per round and not once per token.
 template <typename T, int ND>
 __global__ void __launch_bounds__(64)
 wkv_kernel(float* __restrict__ out, const T* __restrict__ rkv, int64_t plane, const T* __restrict__ z,
            const float* __restrict__ w0, const float* __restrict__ u, float* __restrict__ state,
            const int* __restrict__ cu_q, const int* __restrict__ positions, const int* __restrict__ slots, int H, int D) {
   __shared__ float4 stage[kRound * ND];  // (r, k, w, u k) per (token of the round, key channel)
+  __shared__ float vst[kRound * 64];     // the lanes' v per token of the round
   const int s = blockIdx.z, hd = blockIdx.y, lane = threadIdx.x;
   const int col = blockIdx.x * 64 + lane;
   const int q0 = cu_q[s], q1 = cu_q[s + 1];
@@ -81,20 +84,47 @@ wkv_kernel(float* __restrict__ out, const T* __restrict__ rkv, int64_t plane, co
   const T* rp = rkv;
   const T* kp = rkv + plane;
   const T* vp = rkv + 2 * plane;
+  const float* w0h = w0 + hd * D;
+  const float* uh = u + hd * D;
+  constexpr int kPer = kRound * ND / 64;  // (token, key channel) pairs per lane and round
+  constexpr int kChunk = 8;
   for (int t0 = q0; t0 < q1; t0 += kRound) {
     const int nt = min(kRound, q1 - t0);
+    const int n_el = nt * D;
     __syncthreads();
-    for (int e = lane; e < nt * D; e += 64) {
-      const int j = e / D, d = e - j * D;
-      const int64_t at = static_cast<int64_t>(t0 + j) * HD + static_cast<int64_t>(hd) * D + d;
-      const float k = ld<T>(kp + at);
-      const float w = expf(-expf(ld<T>(z + at) + w0[hd * D + d]));
-      stage[j * ND + d] = float4{ld<T>(rp + at), k, w, u[hd * D + d] * k};
+    for (int c0 = 0; c0 < kPer; c0 += kChunk) {
+      if (c0 * 64 >= n_el) break;
+      float rr[kChunk], kk[kChunk], zz[kChunk];
+#pragma unroll
+      for (int i = 0; i < kChunk; ++i) {
+        const int e = (c0 + i) * 64 + lane;
+        const int j = e / D, d = e - j * D;
+        const int64_t at = static_cast<int64_t>(t0 + j) * HD + static_cast<int64_t>(hd) * D + d;
+        const bool ok = e < n_el;
+        rr[i] = ok ? ld<T>(rp + at) : 0.f;
+        kk[i] = ok ? ld<T>(kp + at) : 0.f;
+        zz[i] = ok ? ld<T>(z + at) : 0.f;
+      }
+#pragma unroll
+      for (int i = 0; i < kChunk; ++i) {
+        const int e = (c0 + i) * 64 + lane;
+        if (e < n_el) {
+          const int j = e / D, d = e - j * D;
+          stage[j * ND + d] = float4{rr[i], kk[i], expf(-expf(zz[i] + w0h[d])), uh[d] * kk[i]};
+        }
+      }
+    }
+    {
+      float tv[kRound];
+#pragma unroll
+      for (int j = 0; j < kRound; ++j)
+        tv[j] = (live && j < nt) ? ld<T>(vp + static_cast<int64_t>(t0 + j) * HD + static_cast<int64_t>(hd) * D + col) : 0.f;
+#pragma unroll
+      for (int j = 0; j < kRound; ++j) vst[j * 64 + lane] = tv[j];
     }
     __syncthreads();
     for (int j = 0; j < nt; ++j) {
-      const int64_t at = static_cast<int64_t>(t0 + j) * HD + static_cast<int64_t>(hd) * D + col;
-      const float vv = live ? ld<T>(vp + at) : 0.f;
+      const float vv = vst[j * 64 + lane];
       float o = 0.f;
 #pragma unroll
       for (int d = 0; d < ND; ++d) {
@@ -104,7 +134,7 @@ wkv_kernel(float* __restrict__ out, const T* __restrict__ rkv, int64_t plane, co
           S[d] = f.z * S[d] + f.y * vv;
         }
       }
-      if (live) out[at] = o;
+      if (live) out[static_cast<int64_t>(t0 + j) * HD + static_cast<int64_t>(hd) * D + col] = o;
     }
   }
   if (sp && live) {
