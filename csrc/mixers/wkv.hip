@@ -6,10 +6,10 @@
 //   tanh        in place
 //   wkv         per (sequence, head), state S [D, D] fp32 (key channel, value channel):
 //                 w_t = exp(-exp(z_t + w0));  o_t = (S + diag(u) k_t v_t^T)^T r_t;  S <- diag(w_t) S + k_t v_t^T
-//               A wave owns 64 value columns of a (sequence, head); every lane keeps its column of S in
-//               registers; r, k, w and u k of a round of 16 tokens are staged in LDS (one 16-byte
-//               broadcast read per key channel).  Tokens are walked in order with the same order of
-//               sums whether a token arrives in a portion or alone.
+//               A workgroup owns 64 value columns of a (sequence, head); its waves share the key
+//               channels of every column's state, kept in registers; r, k, w and u k of a round of 16
+//               tokens are staged in LDS (one 16-byte broadcast read per key channel).  Tokens are
+//               walked in order with the same order of sums whether a token arrives in a portion or alone.
 #include "mix_common.h"
 
 using namespace pkm;
@@ -59,45 +59,48 @@ __global__ void __launch_bounds__(256) tanh_kernel(T* __restrict__ x, int64_t n)
 
 constexpr int kRound = 16;  // tokens staged per round
 
-// ND: key channels kept per lane (>= D).  grid (column groups of 64, H, sequences), one wave each.
-// A round's loads (r, k, z of every key channel, the lane's v of every token) are issued together
-// before their first use, so the wave waits for memory once per round and not once per token.
-template <typename T, int ND>
-__global__ void __launch_bounds__(64)
+// A workgroup of NW waves owns 64 value columns of a (sequence, head); wave w keeps key channels
+// w NR .. w NR + NR - 1 of every column's state in registers (NR NW >= D).  Per round of 16 tokens
+// the workgroup stages (r, k, w, u k) of every key channel and v of its columns in LDS with all loads
+// issued together, every wave walks the round's tokens over its key channels, and the waves' partial
+// outputs are summed in wave order.  grid (column groups of 64, H, sequences).
+template <typename T, int NR, int NW>
+__global__ void __launch_bounds__(64 * NW)
 wkv_kernel(float* __restrict__ out, const T* __restrict__ rkv, int64_t plane, const T* __restrict__ z,
            const float* __restrict__ w0, const float* __restrict__ u, float* __restrict__ state,
            const int* __restrict__ cu_q, const int* __restrict__ positions, const int* __restrict__ slots, int H, int D) {
-  __shared__ float4 stage[kRound * ND];  // (r, k, w, u k) per (token of the round, key channel)
-  __shared__ float vst[kRound * 64];     // the lanes' v per token of the round
-  const int s = blockIdx.z, hd = blockIdx.y, lane = threadIdx.x;
+  constexpr int ND = NR * NW, kThreads = 64 * NW;
+  __shared__ float4 stage[kRound * ND];       // (r, k, w, u k) per (token of the round, key channel)
+  __shared__ float vst[kRound * 64];          // the columns' v per token of the round
+  __shared__ float part[NW * kRound * 64];    // the waves' partial outputs
+  const int s = blockIdx.z, hd = blockIdx.y, tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
   const int col = blockIdx.x * 64 + lane;
   const int q0 = cu_q[s], q1 = cu_q[s + 1];
   if (q1 <= q0) return;
   const int slot = slots[s];
   const int64_t HD = static_cast<int64_t>(H) * D;
   const bool live = col < D;
-  float S[ND];
+  const int d0 = w * NR;
+  float S[NR];
   float* sp = slot >= 0 ? state + (static_cast<int64_t>(slot) * H + hd) * D * D + col : nullptr;
   const bool carry = sp != nullptr && positions[q0] > 0;
 #pragma unroll
-  for (int d = 0; d < ND; ++d) S[d] = (carry && live && d < D) ? sp[static_cast<int64_t>(d) * D] : 0.f;
+  for (int i = 0; i < NR; ++i) S[i] = (carry && live && d0 + i < D) ? sp[static_cast<int64_t>(d0 + i) * D] : 0.f;
   const T* rp = rkv;
   const T* kp = rkv + plane;
   const T* vp = rkv + 2 * plane;
   const float* w0h = w0 + hd * D;
   const float* uh = u + hd * D;
-  constexpr int kPer = kRound * ND / 64;  // (token, key channel) pairs per lane and round
-  constexpr int kChunk = 8;
+  constexpr int kPer = kRound * ND / kThreads;  // (token, key channel) pairs per thread and round
   for (int t0 = q0; t0 < q1; t0 += kRound) {
     const int nt = min(kRound, q1 - t0);
     const int n_el = nt * D;
     __syncthreads();
-    for (int c0 = 0; c0 < kPer; c0 += kChunk) {
-      if (c0 * 64 >= n_el) break;
-      float rr[kChunk], kk[kChunk], zz[kChunk];
+    {
+      float rr[kPer], kk[kPer], zz[kPer];
 #pragma unroll
-      for (int i = 0; i < kChunk; ++i) {
-        const int e = (c0 + i) * 64 + lane;
+      for (int i = 0; i < kPer; ++i) {
+        const int e = i * kThreads + tid;
         const int j = e / D, d = e - j * D;
         const int64_t at = static_cast<int64_t>(t0 + j) * HD + static_cast<int64_t>(hd) * D + d;
         const bool ok = e < n_el;
@@ -105,42 +108,49 @@ wkv_kernel(float* __restrict__ out, const T* __restrict__ rkv, int64_t plane, co
         kk[i] = ok ? ld<T>(kp + at) : 0.f;
         zz[i] = ok ? ld<T>(z + at) : 0.f;
       }
+      float tv[kRound / NW];
 #pragma unroll
-      for (int i = 0; i < kChunk; ++i) {
-        const int e = (c0 + i) * 64 + lane;
+      for (int i = 0; i < kRound / NW; ++i) {
+        const int j = w + i * NW;
+        tv[i] = (live && j < nt) ? ld<T>(vp + static_cast<int64_t>(t0 + j) * HD + static_cast<int64_t>(hd) * D + col) : 0.f;
+      }
+#pragma unroll
+      for (int i = 0; i < kPer; ++i) {
+        const int e = i * kThreads + tid;
         if (e < n_el) {
           const int j = e / D, d = e - j * D;
           stage[j * ND + d] = float4{rr[i], kk[i], expf(-expf(zz[i] + w0h[d])), uh[d] * kk[i]};
         }
       }
-    }
-    {
-      float tv[kRound];
 #pragma unroll
-      for (int j = 0; j < kRound; ++j)
-        tv[j] = (live && j < nt) ? ld<T>(vp + static_cast<int64_t>(t0 + j) * HD + static_cast<int64_t>(hd) * D + col) : 0.f;
-#pragma unroll
-      for (int j = 0; j < kRound; ++j) vst[j * 64 + lane] = tv[j];
+      for (int i = 0; i < kRound / NW; ++i) vst[(w + i * NW) * 64 + lane] = tv[i];
     }
     __syncthreads();
     for (int j = 0; j < nt; ++j) {
       const float vv = vst[j * 64 + lane];
       float o = 0.f;
 #pragma unroll
-      for (int d = 0; d < ND; ++d) {
-        if (d < D) {
-          const float4 f = stage[j * ND + d];
-          o += f.x * (S[d] + f.w * vv);
-          S[d] = f.z * S[d] + f.y * vv;
+      for (int i = 0; i < NR; ++i) {
+        if (d0 + i < D) {
+          const float4 f = stage[j * ND + d0 + i];
+          o += f.x * (S[i] + f.w * vv);
+          S[i] = f.z * S[i] + f.y * vv;
         }
       }
+      part[(w * kRound + j) * 64 + lane] = o;
+    }
+    __syncthreads();
+    for (int j = w; j < nt; j += NW) {
+      float o = 0.f;
+#pragma unroll
+      for (int ww = 0; ww < NW; ++ww) o += part[(ww * kRound + j) * 64 + lane];
       if (live) out[static_cast<int64_t>(t0 + j) * HD + static_cast<int64_t>(hd) * D + col] = o;
     }
   }
   if (sp && live) {
 #pragma unroll
-    for (int d = 0; d < ND; ++d)
-      if (d < D) sp[static_cast<int64_t>(d) * D] = S[d];
+    for (int i = 0; i < NR; ++i)
+      if (d0 + i < D) sp[static_cast<int64_t>(d0 + i) * D] = S[i];
   }
 }
 
@@ -180,20 +190,20 @@ PK_EXPORT int pkm_wkv(void* out, const void* rkv, long long plane, const void* z
   if (T <= 0 || n_seqs <= 0) return 0;
   if (H < 1 || D < 1 || D > 256) return -1;
   const dim3 grid((D + 63) / 64, H, n_seqs);
-#define PKM_WKV(ND)                                                                                                     \
-  PKM_DISPATCH(dt, E, wkv_kernel<E, ND><<<grid, 64, 0, stream>>>(                                                          \
+#define PKM_WKV(NR, NW)                                                                                                 \
+  PKM_DISPATCH(dt, E, wkv_kernel<E, NR, NW><<<grid, 64 * NW, 0, stream>>>(                                                 \
                           static_cast<float*>(out), static_cast<const E*>(rkv), plane, static_cast<const E*>(z),           \
                           static_cast<const float*>(w0), static_cast<const float*>(u), static_cast<float*>(state),         \
                           static_cast<const int*>(cu_q), static_cast<const int*>(positions), static_cast<const int*>(slots), \
                           H, D))
   if (D <= 32) {
-    PKM_WKV(32);
+    PKM_WKV(8, 4);
   } else if (D <= 64) {
-    PKM_WKV(64);
+    PKM_WKV(16, 4);
   } else if (D <= 128) {
-    PKM_WKV(128);
+    PKM_WKV(32, 4);
   } else {
-    PKM_WKV(256);
+    PKM_WKV(32, 8);
   }
 #undef PKM_WKV
   return PK_CHECK_LAUNCH();
