@@ -125,7 +125,7 @@ def pooled_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
     # few row tiles (decoded tokens): the key tiles of a row tile are dealt to several workgroups and merged
     tiles = (-(-T * rep // 16) + n_seqs) * G
     span = block_tables.shape[1] * bs if window <= 0 else min(block_tables.shape[1] * bs, window + 64)
-    n_parts = max(1, min(16, 2048 // tiles, span // 64))
+    n_parts = max(1, min(16, 1024 // tiles, span // 64))
     ws_acc = ws_ml = None
     if n_parts > 1:
         ws_acc = torch.empty((T * H, n_parts, VG * V), dtype=torch.float32, device=q.device)
