@@ -329,6 +329,240 @@ __global__ void __launch_bounds__(kThreads) pooled_attention_kernel(PooledArgs a
   }
 }
 
+// ---- bf16 on the matrix cores -------------------------------------------------------------------
+// The same tile problem (16 (token, head) rows of one key head against 32-key tiles, block means first) with
+// both products on mfma_f32_16x16x32_bf16.  Lane (g, n) = (lane / 16, lane % 16) supplies A[row n][k 8g..8g+7]
+// and B[k 8g..8g+7][column n] and holds C[rows 4g..4g+3][column n].
+//   S [rows x keys]  = Q [rows x D] . K^T       A = query rows, B = key rows, both 16-byte reads of bf16 LDS tiles
+//   O [rows x cols] += P [rows x keys] . V      A = the softmax weights rounded to bf16, B = a value column's 8 keys
+// Tiles are staged as they lie in the cache (16-byte copies, no conversion).  Wave w takes the 16-key blocks
+// w, w + 4, .. of the first product and the 16-column blocks w, w + 4, .. of the second; cap, band, sink and the
+// running maximum / sum stay with the 16 x 16 thread layout of the FMA kernel.
+template <int NV>
+__global__ void __launch_bounds__(kThreads) pooled_attention_mfma_kernel(PooledArgs a) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  const int H = a.H, G = a.G, D = a.D, V = a.V, BK = a.BK, bs = a.bs;
+  const int R = H / G;
+  const int kh = blockIdx.y;
+  const int VG = a.all_values ? G : 1;
+  const int VW = VG * V;
+  int s = 0, tile = blockIdx.x;
+  for (; s < a.n_seqs; ++s) {
+    const int rows = (a.cu_q[s + 1] - a.cu_q[s]) * R;
+    const int nt = (rows + kBQ - 1) / kBQ;
+    if (tile < nt) break;
+    tile -= nt;
+  }
+  if (s >= a.n_seqs) return;
+  const int q0 = a.cu_q[s], qlen = a.cu_q[s + 1] - q0, ctx = a.context_lens[s];
+  const int n_rows = qlen * R;
+  const int row0 = tile * kBQ;
+  const int DSH = D + 8, VSH = VW + 8, PSH = BK + 8;  // bf16 row strides: rows stay 16-byte aligned, banks shift
+  bf16_t* qs = reinterpret_cast<bf16_t*>(smem_raw);  // [kBQ][DSH]
+  bf16_t* ks = qs + kBQ * DSH;                       // [BK][DSH]
+  bf16_t* vs = ks + BK * DSH;                        // [BK][VSH]
+  bf16_t* pb = vs + BK * VSH;                        // [kBQ][PSH] softmax weights as bf16
+  float* ps = reinterpret_cast<float*>(pb + kBQ * PSH);  // [kBQ][BK] scores, then weights
+  float* m_s = ps + kBQ * BK;
+  float* l_s = m_s + kBQ;
+  float* r_s = l_s + kBQ;
+  const int tid = threadIdx.x;
+  const int qi = tid >> 4, kg = tid & 15;
+  const int lane = tid & 63, w = tid >> 6, g4 = lane >> 4, n = lane & 15;
+  const int* bt = a.block_tables + static_cast<int64_t>(s) * a.bt_stride;
+  const uint4 zero4 = uint4{0u, 0u, 0u, 0u};
+
+  for (int u = tid; u < kBQ * (D / 8); u += kThreads) {
+    const int r = u / (D / 8), c = (u - r * (D / 8)) * 8;
+    const int row = row0 + r;
+    uint4 v = zero4;
+    if (row < n_rows) {
+      const int tl = row / R, h = kh * R + row - tl * R;
+      v = *reinterpret_cast<const uint4*>(static_cast<const bf16_t*>(a.q) + (static_cast<int64_t>(q0 + tl) * H + h) * D + c);
+    }
+    *reinterpret_cast<uint4*>(qs + r * DSH + c) = v;
+  }
+  const int my_row = row0 + qi;
+  const bool live = my_row < n_rows;
+  const int my_tl = live ? my_row / R : 0;
+  const int my_pos = live ? ctx - qlen + my_tl : -1;
+  const int my_lo = (live && a.window > 0) ? max(0, my_pos - a.window + 1) : 0;
+  const int my_blocks = live ? blocks_seen(my_pos, a.window, a.pool) : 0;
+  if (tid < kBQ) {
+    const int row = row0 + tid;
+    const int h = kh * R + (row < n_rows ? row % R : 0);
+    const bool sink_here = a.sink && a.n_parts <= 1;
+    m_s[tid] = sink_here ? a.sink[h] : -INFINITY;
+    l_s[tid] = sink_here ? 1.f : 0.f;
+  }
+  const int first_pos = ctx - qlen + row0 / R;
+  const int last_pos = ctx - qlen + (min(row0 + kBQ, n_rows) - 1) / R;
+  pk::f32x4 acc[NV];
+#pragma unroll
+  for (int i = 0; i < NV; ++i) acc[i] = pk::f32x4{0.f, 0.f, 0.f, 0.f};
+  __syncthreads();
+
+  int tile_no = 0;
+  for (int part = 0; part < 2; ++part) {
+    const bf16_t* kc = static_cast<const bf16_t*>(part ? a.k_cache : a.kp_cache);
+    const bf16_t* vc = static_cast<const bf16_t*>(part ? a.v_cache : a.vp_cache);
+    int k_begin, k_end;
+    if (part == 0) {
+      k_begin = 0;
+      k_end = last_pos >= 0 ? blocks_seen(last_pos, a.window, a.pool) : 0;
+    } else {
+      k_end = last_pos + 1;
+      k_begin = (first_pos >= 0 && a.window > 0) ? max(0, first_pos - a.window + 1) / BK * BK : 0;
+    }
+    for (int k0 = k_begin; k0 < k_end; k0 += BK) {
+      if (a.n_parts > 1 && (tile_no++) % a.n_parts != static_cast<int>(blockIdx.z)) continue;
+      const int nk = min(BK, k_end - k0);
+      {  // key rows, then the value rows of the staged value heads: 16-byte copies, four per thread and pass
+        const int kper = D / 8, vper = VW / 8;
+        const int units = BK * (kper + vper);
+        for (int u0 = 0; u0 < units; u0 += 4 * kThreads) {
+          uint4 v[4];
+#pragma unroll
+          for (int p = 0; p < 4; ++p) {
+            const int u = u0 + p * kThreads + tid;
+            v[p] = zero4;
+            if (u < BK * kper) {
+              const int j = u / kper, c = (u - j * kper) * 8;
+              if (j < nk) {
+                const int key = k0 + j;
+                v[p] = *reinterpret_cast<const uint4*>(kc + ((static_cast<int64_t>(bt[key / bs]) * G + kh) * bs + key % bs) * D + c);
+              }
+            } else if (u < units) {
+              const int u2 = u - BK * kper;
+              const int j = u2 / vper, c = (u2 - j * vper) * 8;
+              if (j < nk) {
+                const int key = k0 + j;
+                const int g = a.all_values ? c / V : kh, cc = a.all_values ? c - g * V : c;
+                v[p] = *reinterpret_cast<const uint4*>(vc + ((static_cast<int64_t>(bt[key / bs]) * G + g) * bs + key % bs) * V + cc);
+              }
+            }
+          }
+#pragma unroll
+          for (int p = 0; p < 4; ++p) {
+            const int u = u0 + p * kThreads + tid;
+            if (u < BK * kper) {
+              const int j = u / kper, c = (u - j * kper) * 8;
+              *reinterpret_cast<uint4*>(ks + j * DSH + c) = v[p];
+            } else if (u < units) {
+              const int u2 = u - BK * kper;
+              const int j = u2 / vper, c = (u2 - j * vper) * 8;
+              *reinterpret_cast<uint4*>(vs + j * VSH + c) = v[p];
+            }
+          }
+        }
+      }
+      __syncthreads();
+      for (int kb = w; kb < BK / 16; kb += kThreads / 64) {
+        pk::f32x4 c4 = pk::f32x4{0.f, 0.f, 0.f, 0.f};
+        const bf16_t* qr = qs + n * DSH + 8 * g4;
+        const bf16_t* kr = ks + (kb * 16 + n) * DSH + 8 * g4;
+        for (int kk = 0; kk < D / 32; ++kk)
+          c4 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pk::ld8(qr + kk * 32), pk::ld8(kr + kk * 32), c4, 0, 0, 0);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) ps[(4 * g4 + i) * BK + kb * 16 + n] = c4[i];
+      }
+      __syncthreads();
+      float tmax = -INFINITY;
+      for (int j = kg; j < BK; j += 16) {
+        const int key = k0 + j;
+        const bool seen = j < nk && live && (part == 0 ? key < my_blocks : (key <= my_pos && key >= my_lo));
+        float d = -INFINITY;
+        if (seen) {
+          d = ps[qi * BK + j] * a.scale;
+          if (a.softcap > 0.f) d = a.softcap * tanhf(d / a.softcap);
+        }
+        ps[qi * BK + j] = d;
+        tmax = fmaxf(tmax, d);
+      }
+#pragma unroll
+      for (int o = 8; o > 0; o >>= 1) tmax = fmaxf(tmax, __shfl_xor(tmax, o, 64));
+      const float m_old = m_s[qi];
+      const float m_new = fmaxf(m_old, tmax);
+      float tsum = 0.f;
+      for (int j = kg; j < BK; j += 16) {
+        const float sc = ps[qi * BK + j];
+        const float p = (m_new == -INFINITY || sc == -INFINITY) ? 0.f : expf(sc - m_new);
+        pb[qi * PSH + j] = pk::f2bf(p);
+        tsum += p;
+      }
+#pragma unroll
+      for (int o = 8; o > 0; o >>= 1) tsum += __shfl_xor(tsum, o, 64);
+      const float resc = (m_old == -INFINITY) ? 0.f : expf(m_old - m_new);
+      if (kg == 0) r_s[qi] = resc;
+      __syncthreads();
+      if (kg == 0) {
+        m_s[qi] = m_new;
+        l_s[qi] = l_s[qi] * resc + tsum;
+      }
+      {
+        float rs[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) rs[e] = r_s[4 * g4 + e];
+#pragma unroll
+        for (int i = 0; i < NV; ++i)
+#pragma unroll
+          for (int e = 0; e < 4; ++e) acc[i][e] *= rs[e];
+        for (int k32 = 0; k32 < BK / 32; ++k32) {
+          const pk::bf16x8_t pa = pk::ld8(pb + n * PSH + k32 * 32 + 8 * g4);
+#pragma unroll
+          for (int i = 0; i < NV; ++i) {
+            const int col = (w + 4 * i) * 16 + n;
+            if ((w + 4 * i) * 16 < VW) {
+              const bf16_t* vr = vs + (k32 * 32 + 8 * g4) * VSH + col;
+              pk::u32x4 bw;
+#pragma unroll
+              for (int e = 0; e < 4; ++e)
+                bw[e] = static_cast<uint32_t>(vr[(2 * e) * VSH]) | (static_cast<uint32_t>(vr[(2 * e + 1) * VSH]) << 16);
+              acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pa, __builtin_bit_cast(pk::bf16x8_t, bw), acc[i], 0, 0, 0);
+            }
+          }
+        }
+      }
+      __syncthreads();
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const int row = row0 + 4 * g4 + e;
+    if (row >= n_rows) break;
+    const int tl = row / R, h = kh * R + row - tl * R;
+    const float l = l_s[4 * g4 + e];
+    if (a.n_parts > 1) {
+      const int64_t slot = (static_cast<int64_t>(q0 + tl) * H + h) * a.n_parts + blockIdx.z;
+      float* dst = a.ws_acc + slot * VW;
+#pragma unroll
+      for (int i = 0; i < NV; ++i) {
+        const int c = (w + 4 * i) * 16 + n;
+        if (c < VW) dst[c] = acc[i][e];
+      }
+      if (w == 0 && n == 0) {
+        a.ws_ml[2 * slot] = m_s[4 * g4 + e];
+        a.ws_ml[2 * slot + 1] = l;
+      }
+    } else {
+      const float inv = l > 0.f ? 1.f / l : 0.f;
+      float* dst = a.out + (static_cast<int64_t>(q0 + tl) * H + h) * VW;
+#pragma unroll
+      for (int i = 0; i < NV; ++i) {
+        const int c = (w + 4 * i) * 16 + n;
+        if (c < VW) dst[c] = acc[i][e] * inv;
+      }
+    }
+  }
+}
+
+size_t mfma_lds_bytes(int D, int VW, int bk) {
+  return (static_cast<size_t>(kBQ) * (D + 8) + static_cast<size_t>(bk) * (D + 8 + VW + 8) + kBQ * (bk + 8)) * 2 +
+         (static_cast<size_t>(kBQ) * bk + 3 * kBQ) * 4;
+}
+
+int g_pooled_mfma = 1;  // 0: every launch takes the FMA kernel (tests compare the two)
+
 // out[t, h] from the parts' (max, sum, unnormalised sums) and the head's sink: one wave per (token, head)
 __global__ void __launch_bounds__(64)
 pooled_merge_kernel(float* __restrict__ out, const float* __restrict__ ws_acc, const float* __restrict__ ws_ml,
@@ -447,11 +681,35 @@ PK_EXPORT int pkm_pooled_attention(void* out, const void* q, const void* k_cache
   const int tiles = (T * R + kBQ - 1) / kBQ + n_seqs;
   const dim3 grid(tiles, G, n_parts);
   int rc = -2;
-  if (dt == kBF16) rc = launch_pooled<bf16_t>(a, grid, VW, stream);
+  // bf16 with sizes the matrix-core tiles take: 32-key tiles within the default LDS limit
+  if (dt == kBF16 && g_pooled_mfma && D % 32 == 0 && V % 8 == 0 && VW % 16 == 0 && mfma_lds_bytes(D, VW, 32) <= 60 * 1024) {
+    a.BK = 32;
+    const size_t lds = mfma_lds_bytes(D, VW, 32);
+    const int nv = (VW + 63) / 64;
+#define PKM_PM(NV) pooled_attention_mfma_kernel<NV><<<grid, kThreads, lds, stream>>>(a)
+    if (nv <= 1) {
+      PKM_PM(1);
+    } else if (nv <= 2) {
+      PKM_PM(2);
+    } else if (nv <= 4) {
+      PKM_PM(4);
+    } else if (nv <= 8) {
+      PKM_PM(8);
+    } else {
+      PKM_PM(16);
+    }
+#undef PKM_PM
+    rc = PK_CHECK_LAUNCH();
+  } else if (dt == kBF16) rc = launch_pooled<bf16_t>(a, grid, VW, stream);
   if (dt == kF32) rc = launch_pooled<float>(a, grid, VW, stream);
   if (rc != 0 || n_parts == 1) return rc;
   pooled_merge_kernel<<<dim3(T, H), 64, 0, stream>>>(a.out, a.ws_acc, a.ws_ml, a.sink, H, VW, n_parts);
   return PK_CHECK_LAUNCH();
+}
+
+PK_EXPORT int pkm_set_pooled_mfma(int on) {
+  g_pooled_mfma = on;
+  return 0;
 }
 
 // o fp32 [T, H, VG, V]; talk [H, H] fp32 (VG = G) or null (VG = 1); out rows out_stride elements apart

@@ -125,6 +125,7 @@ MIXER_SIGNATURES = {
     "pkm_pooled_attention": [P, P, P, P, P, P, P, I64, P, P, P, I32, I32, I32, I32, I32, I32, I32, F32, F32, I32, I32, I32,
                              I32, P, P, I32, P],
     "pkm_mix_heads": [P, I64, I32, P, P, I32, I32, I32, I32, F32, P],
+    "pkm_set_pooled_mfma": [I32],
 }
 _mixers: Optional[ctypes.CDLL] = None
 

@@ -647,3 +647,46 @@ def test_aligned_sizes_in_mixed_batches_with_decode_graphs(tmp_path):
         g, r = rows_of(got, rid, n).cpu(), rows_of(ref, rid, n)
         assert float(rel(g, r).mean()) < 0.03, rid
         assert float(rel(g, logits_of(cfg, w, toks[rid]).float()).median()) < 0.1, rid
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("H,G,D,V,window,pool,talk", [(4, 2, 64, 64, 100, 16, True), (8, 2, 128, 128, 70, 7, True), (2, 2, 32, 8, 0, 0, False),
+                                                      (6, 3, 96, 40, 33, 33, True), (16, 4, 128, 128, 200, 64, True)])
+def test_matrix_core_attention_matches_the_fma_tiles(H, G, D, V, window, pool, talk):
+    """bf16 at sizes the matrix-core kernel takes: prompt portions and decoded tokens (their key tiles cut into runs
+    and merged) against the FMA kernel on the same caches, and against the plain rule."""
+    from polykey_service_amd.ops import native
+    from polykey_service_amd.ops import pooled_attention as pa
+    dev, n = torch.device("cuda"), 300
+    g = torch.Generator().manual_seed(H * 100 + D)
+    bf = torch.bfloat16
+    q = torch.randn((n, H, D), generator=g).to(bf)
+    k = (0.5 * torch.randn((n, G, D), generator=g)).to(bf)
+    v = torch.randn((n, G, V), generator=g).to(bf)
+    sink = torch.randn(H, generator=g)
+    tk = (torch.eye(H) + 0.2 * torch.randn((H, H), generator=g)) if talk else None
+    pages = [7, 2, 11, 0, 5, 9, 3, 1, 10, 4, 6, 8]
+    outs = {}
+    for mfma in (1, 0):
+        native.mixers().pkm_set_pooled_mfma(mfma)
+        try:
+            kc, vc = torch.zeros((12, G, BS, D), device=dev, dtype=bf), torch.zeros((12, G, BS, V), device=dev, dtype=bf)
+            kp, vp = torch.full_like(kc, 9.0), torch.full_like(vc, 9.0)
+            feed, got = Feed(dev, pages), []
+            for c in [150, 1, 1, 40, 2, 1, 1, 1, 103]:
+                pos, md = feed.step(c)
+                sl = md.slot_mapping.long()
+                kc[sl // BS, :, sl % BS] = k[feed.at - c:feed.at].to(dev)
+                vc[sl // BS, :, sl % BS] = v[feed.at - c:feed.at].to(dev)
+                pa.pool_update(kc, vc, kp, vp, pos, md.token_seq, md.block_tables, pool, md.slot_mapping)
+                o = pa.pooled_attention(q[feed.at - c:feed.at].contiguous().to(dev), kc, vc, kp, vp, md.block_tables, md.cu_q,
+                                        md.context_lens, 1, D ** -0.5, 12.0, window, pool, sink.to(dev), all_values=talk)
+                got.append(pa.mix_heads(o, None if tk is None else tk.to(dev), 1.0, torch.float32).cpu())
+            outs[mfma] = torch.cat(got).view(n, H, V)
+        finally:
+            native.mixers().pkm_set_pooled_mfma(1)
+    # the block means are rounded to bf16 in the cache; the plain rule keeps them exact
+    want = O.pooled_softmax(q.double(), k.double(), v.double(), D ** -0.5, 12.0, window, pool, sink.double(),
+                            None if tk is None else tk.double())
+    close(outs[1], outs[0], 2e-2)
+    close(outs[1], want, 4e-2)
