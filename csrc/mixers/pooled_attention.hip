@@ -682,11 +682,19 @@ PK_EXPORT int pkm_pooled_attention(void* out, const void* q, const void* k_cache
   const dim3 grid(tiles, G, n_parts);
   int rc = -2;
   // bf16 with sizes the matrix-core tiles take: 32-key tiles within the default LDS limit
-  if (dt == kBF16 && g_pooled_mfma && D % 32 == 0 && V % 8 == 0 && VW % 16 == 0 && mfma_lds_bytes(D, VW, 32) <= 60 * 1024) {
+  if (dt == kBF16 && g_pooled_mfma && D % 32 == 0 && V % 8 == 0 && VW % 16 == 0 && mfma_lds_bytes(D, VW, 32) <= 144 * 1024) {
     a.BK = 32;
     const size_t lds = mfma_lds_bytes(D, VW, 32);
     const int nv = (VW + 63) / 64;
-#define PKM_PM(NV) pooled_attention_mfma_kernel<NV><<<grid, kThreads, lds, stream>>>(a)
+#define PKM_PM(NV)                                                                                                       \
+  {                                                                                                                      \
+    if (lds > 60 * 1024) {                                                                                               \
+      const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(pooled_attention_mfma_kernel<NV>),          \
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds));        \
+      if (e != hipSuccess) return static_cast<int>(e);                                                                   \
+    }                                                                                                                    \
+    pooled_attention_mfma_kernel<NV><<<grid, kThreads, lds, stream>>>(a);                                                \
+  }
     if (nv <= 1) {
       PKM_PM(1);
     } else if (nv <= 2) {
