@@ -642,17 +642,26 @@ class BibezenConfig:
         return True     # every mixer keeps per-sequence state (filters, previous rows, recurrences)
 
     def num_params(self) -> int:
-        W, n = self.hidden_size, self.vocab_size * self.hidden_size
-        wkv = lambda m: W * m.heads * m.dim * 5 + 2 * max(m.decay_rank, 1) * (W + m.heads * m.dim) // 2
-        att = lambda m: W * (2 * m.heads * m.dim + m.kv_heads * (m.dim + m.vdim)) + W * m.heads * (m.vdim - m.dim)
+        W, n = self.hidden_size, self.vocab_size * self.hidden_size + self.hidden_size
+
+        def wkv(m, own_output=True):
+            c, r = m.heads * m.dim, m.decay_rank or max(16, W // 64)
+            return (5 if own_output else 4) * c * W + r * (W + c) + 5 * W + 3 * c
+
+        def left(m):
+            c = (m.heads + m.kv_heads) * m.dim + m.kv_heads * m.vdim
+            return c * (W + 1 + max(m.conv, 0)) + 2 * m.dim + m.heads * (m.heads + 1) + W * m.heads * m.vdim
+
         for l in self.layers:
             m = l.mixer
+            n += W * (2 if l.mlp is not None else 1) + max(self.streams, 0) * (self.streams + 2) * (2 if l.mlp is not None else 1)
+            n += W * self.canon_taps
             if l.type == "wkv":
                 n += wkv(m)
             elif l.type == "mamba1":
-                n += 3 * W * m.inner + m.inner * (m.dt_rank * 2 + 2 * m.state) + m.inner * m.state
+                n += 3 * W * m.inner + m.inner * (m.conv + 3 + m.state + 2 * m.dt_rank + 2 * m.state)
             else:
-                n += wkv(m.right) + att(m.left)
+                n += left(m.left) + wkv(m.right, False) + W * m.right.heads * m.right.dim
             f = l.mlp
             if isinstance(f, ClampedFFSpec):
                 n += 3 * W * f.ff
