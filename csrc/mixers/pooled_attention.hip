@@ -334,7 +334,8 @@ __global__ void __launch_bounds__(kThreads) pooled_attention_kernel(PooledArgs a
 // both products on mfma_f32_16x16x32_bf16.  Lane (g, n) = (lane / 16, lane % 16) supplies A[row n][k 8g..8g+7]
 // and B[k 8g..8g+7][column n] and holds C[rows 4g..4g+3][column n].
 //   S [rows x keys]  = Q [rows x D] . K^T       A = query rows, B = key rows, both 16-byte reads of bf16 LDS tiles
-//   O [rows x cols] += P [rows x keys] . V      A = the softmax weights rounded to bf16, B = a value column's 8 keys
+//   O [rows x cols] += P [rows x keys] . V      A = the softmax weights as two bf16 parts (leading part and
+//                                               remainder, two instructions), B = a value column's 8 keys
 // Tiles are staged as they lie in the cache (16-byte copies, no conversion).  Wave w takes the 16-key blocks
 // w, w + 4, .. of the first product and the 16-column blocks w, w + 4, .. of the second; cap, band, sink and the
 // running maximum / sum stay with the 16 x 16 thread layout of the FMA kernel.
@@ -361,8 +362,9 @@ __global__ void __launch_bounds__(kThreads) pooled_attention_mfma_kernel(PooledA
   bf16_t* qs = reinterpret_cast<bf16_t*>(smem_raw);  // [kBQ][DSH]
   bf16_t* ks = qs + kBQ * DSH;                       // [BK][DSH]
   bf16_t* vs = ks + BK * DSH;                        // [BK][VSH]
-  bf16_t* pb = vs + BK * VSH;                        // [kBQ][PSH] softmax weights as bf16
-  float* ps = reinterpret_cast<float*>(pb + kBQ * PSH);  // [kBQ][BK] scores, then weights
+  bf16_t* pb = vs + BK * VSH;                        // [2][kBQ][PSH] softmax weights as bf16: leading part, remainder
+  bf16_t* pb2 = pb + kBQ * PSH;
+  float* ps = reinterpret_cast<float*>(pb2 + kBQ * PSH);  // [kBQ][BK] scores, then weights
   float* m_s = ps + kBQ * BK;
   float* l_s = m_s + kBQ;
   float* r_s = l_s + kBQ;
@@ -487,7 +489,9 @@ __global__ void __launch_bounds__(kThreads) pooled_attention_mfma_kernel(PooledA
       for (int j = kg; j < BK; j += 16) {
         const float sc = ps[qi * BK + j];
         const float p = (m_new == -INFINITY || sc == -INFINITY) ? 0.f : expf(sc - m_new);
-        pb[qi * PSH + j] = pk::f2bf(p);
+        const bf16_t hi = pk::f2bf(p);  // p = hi + lo to 16 bits: the weights meet the values at fp32-like precision
+        pb[qi * PSH + j] = hi;
+        pb2[qi * PSH + j] = pk::f2bf(p - pk::bf2f(hi));
         tsum += p;
       }
 #pragma unroll
@@ -509,6 +513,7 @@ __global__ void __launch_bounds__(kThreads) pooled_attention_mfma_kernel(PooledA
           for (int e = 0; e < 4; ++e) acc[i][e] *= rs[e];
         for (int k32 = 0; k32 < BK / 32; ++k32) {
           const pk::bf16x8_t pa = pk::ld8(pb + n * PSH + k32 * 32 + 8 * g4);
+          const pk::bf16x8_t pa2 = pk::ld8(pb2 + n * PSH + k32 * 32 + 8 * g4);
 #pragma unroll
           for (int i = 0; i < NV; ++i) {
             const int col = (w + 4 * i) * 16 + n;
@@ -518,7 +523,9 @@ __global__ void __launch_bounds__(kThreads) pooled_attention_mfma_kernel(PooledA
 #pragma unroll
               for (int e = 0; e < 4; ++e)
                 bw[e] = static_cast<uint32_t>(vr[(2 * e) * VSH]) | (static_cast<uint32_t>(vr[(2 * e + 1) * VSH]) << 16);
-              acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pa, __builtin_bit_cast(pk::bf16x8_t, bw), acc[i], 0, 0, 0);
+              const pk::bf16x8_t vb = __builtin_bit_cast(pk::bf16x8_t, bw);
+              acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pa, vb, acc[i], 0, 0, 0);
+              acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pa2, vb, acc[i], 0, 0, 0);
             }
           }
         }
@@ -557,7 +564,7 @@ __global__ void __launch_bounds__(kThreads) pooled_attention_mfma_kernel(PooledA
 }
 
 size_t mfma_lds_bytes(int D, int VW, int bk) {
-  return (static_cast<size_t>(kBQ) * (D + 8) + static_cast<size_t>(bk) * (D + 8 + VW + 8) + kBQ * (bk + 8)) * 2 +
+  return (static_cast<size_t>(kBQ) * (D + 8) + static_cast<size_t>(bk) * (D + 8 + VW + 8) + 2 * kBQ * (bk + 8)) * 2 +
          (static_cast<size_t>(kBQ) * bk + 3 * kBQ) * 4;
 }
 
