@@ -688,5 +688,5 @@ def test_matrix_core_attention_matches_the_fma_tiles(H, G, D, V, window, pool, t
     # the block means are rounded to bf16 in the cache; the plain rule keeps them exact
     want = O.pooled_softmax(q.double(), k.double(), v.double(), D ** -0.5, 12.0, window, pool, sink.double(),
                             None if tk is None else tk.double())
-    close(outs[1], outs[0], 2e-2)
+    close(outs[1], outs[0], 2e-3)
     close(outs[1], want, 4e-2)
