@@ -651,7 +651,7 @@ def test_aligned_sizes_in_mixed_batches_with_decode_graphs(tmp_path):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("H,G,D,V,window,pool,talk", [(4, 2, 64, 64, 100, 16, True), (8, 2, 128, 128, 70, 7, True), (2, 2, 32, 8, 0, 0, False),
-                                                      (6, 3, 96, 40, 33, 33, True), (16, 4, 128, 128, 200, 64, True), (16, 8, 64, 128, 150, 10, True)])
+                                                      (6, 3, 96, 40, 33, 33, True), (16, 4, 128, 128, 200, 64, True), (16, 8, 64, 128, 150, 10, True), (6, 2, 96, 48, 50, 9, True)])
 def test_matrix_core_attention_matches_the_fma_tiles(H, G, D, V, window, pool, talk):
     """bf16 at sizes the matrix-core kernel takes: prompt portions and decoded tokens (their key tiles cut into runs
     and merged) against the FMA kernel on the same caches, and against the plain rule."""
